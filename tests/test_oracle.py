@@ -1,0 +1,244 @@
+"""Pins for the CPU oracle (no GPU).  The reference holds no golden vectors for the attention path
+(it has no tests directory), so the oracle is pinned by what the mathematics fixes: a float64 closed
+form, the exp/exp2 equivalence of the reference's own two branches, invariants of softmax attention,
+exact integer arithmetic, and exhaustive codec tables."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+
+def _rand(shape, seed, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(shape) * scale).astype(np.float32)
+
+
+def _closed_form_f64(q, k, v, alpha):
+    q, k, v = (x.astype(np.float64) for x in (q, k, v))
+    s = alpha * np.einsum("bmhd,bnhd->bhmn", q, k)
+    s = s - s.max(axis=-1, keepdims=True)
+    p = np.exp(s)
+    p /= p.sum(axis=-1, keepdims=True)
+    return np.einsum("bhmn,bnhd->bmhd", p, v), p
+
+
+@pytest.mark.parametrize("B,S,H,D", [(1, 64, 2, 64), (2, 128, 3, 128), (1, 96, 1, 256), (1, 33, 2, 16)])
+def test_attention_matches_float64_closed_form(B, S, H, D):
+    q, k, v = _rand((B, S, H, D), 1), _rand((B, S, H, D), 2), _rand((B, S, H, D), 3)
+    ref, _ = _closed_form_f64(q, k, v, 1.0 / np.sqrt(D))
+    got = oracle.attention_f32(q, k, v)["O"]
+    assert np.max(np.abs(got - ref)) < 5e-6
+
+
+def test_transposed_operand_or_dropped_scale_would_fail():
+    # a wrong index (K used where V is meant, or a missing 1/sqrt(D)) moves the result by >> 1e-3
+    B, S, H, D = 1, 64, 2, 64
+    q, k, v = _rand((B, S, H, D), 4), _rand((B, S, H, D), 5), _rand((B, S, H, D), 6)
+    good = oracle.attention_f32(q, k, v)["O"]
+    assert np.max(np.abs(good - oracle.attention_f32(q, k, k)["O"])) > 1e-2
+    assert np.max(np.abs(good - oracle.attention_f32(q, k, v, alpha0=1.0)["O"])) > 1e-2
+    assert np.max(np.abs(good - oracle.attention_f32(k, q, v)["O"])) > 1e-2
+
+
+def test_rectangular_seqlens():
+    B, Sq, Skv, H, D = 1, 48, 80, 2, 32
+    q, k, v = _rand((B, Sq, H, D), 7), _rand((B, Skv, H, D), 8), _rand((B, Skv, H, D), 9)
+    ref, _ = _closed_form_f64(q, k, v, 1.0 / np.sqrt(D))
+    assert np.max(np.abs(oracle.attention_f32(q, k, v)["O"] - ref)) < 5e-6
+
+
+def test_exp_and_exp2_branches_agree():
+    # fmha_cutlass.hpp:242-273 vs :274-302
+    q, k, v = _rand((1, 128, 2, 64), 10), _rand((1, 128, 2, 64), 11), _rand((1, 128, 2, 64), 12)
+    a = oracle.attention_f32(q, k, v, use_pow2=False, want_stats=True)
+    b = oracle.attention_f32(q, k, v, use_pow2=True, want_stats=True)
+    assert np.max(np.abs(a["O"] - b["O"])) < 2e-6
+    # the exp2 branch reports the max in the log2 domain (scores * log2e)
+    np.testing.assert_allclose(b["row_max"], a["row_max"] * oracle.LOG2E, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(a["inv_sum"], b["inv_sum"], rtol=1e-5)
+
+
+def test_post_scaling_only_on_pow2_branch():
+    # usePreScaling=false moves alpha0 to "postScaling", which only the exp2 branch applies
+    # (fmha_cutlass.hpp:206-207, 245-247): the exp branch then runs unscaled.
+    q, k, v = _rand((1, 32, 1, 16), 13), _rand((1, 32, 1, 16), 14), _rand((1, 32, 1, 16), 15)
+    pre = oracle.attention_f32(q, k, v, use_pow2=True, use_prescaling=True)["O"]
+    post = oracle.attention_f32(q, k, v, use_pow2=True, use_prescaling=False)["O"]
+    assert np.max(np.abs(pre - post)) < 2e-6
+    unscaled = oracle.attention_f32(q, k, v, use_pow2=False, use_prescaling=False)["O"]
+    ref, _ = _closed_form_f64(q, k, v, 1.0)
+    assert np.max(np.abs(unscaled - ref)) < 5e-6
+
+
+def test_scores_stats_and_probabilities():
+    B, S, H, D = 2, 64, 2, 32
+    q, k, v = _rand((B, S, H, D), 16), _rand((B, S, H, D), 17), _rand((B, S, H, D), 18)
+    r = oracle.attention_f32(q, k, v, want_scores=True, want_stats=True)
+    s64 = np.einsum("bmhd,bnhd->bhmn", q.astype(np.float64), k.astype(np.float64)) / np.sqrt(D)
+    assert np.max(np.abs(r["S"] - s64)) < 1e-5
+    np.testing.assert_allclose(r["row_max"], s64.max(-1), atol=1e-5)
+    z = np.exp(s64 - s64.max(-1, keepdims=True)).sum(-1)
+    np.testing.assert_allclose(r["inv_sum"], 1.0 / z, rtol=1e-5)
+    # rows of P sum to one: V = ones gives O = ones
+    ones = oracle.attention_f32(q, k, np.ones_like(v))["O"]
+    assert np.max(np.abs(ones - 1.0)) < 1e-5
+
+
+def test_invariants():
+    B, S, H, D = 1, 64, 2, 32
+    q, k, v = _rand((B, S, H, D), 19), _rand((B, S, H, D), 20), _rand((B, S, H, D), 21)
+    o = oracle.attention_f32(q, k, v)["O"]
+    # convexity: min_k V <= O <= max_k V per (b,h,d)
+    assert np.all(o <= v.max(axis=1, keepdims=True) + 1e-5) and np.all(o >= v.min(axis=1, keepdims=True) - 1e-5)
+    # Q = 0 -> uniform probabilities -> mean of V
+    o0 = oracle.attention_f32(np.zeros_like(q), k, v)["O"]
+    assert np.max(np.abs(o0 - v.mean(axis=1, keepdims=True))) < 1e-5
+    # key permutation invariance (pins the fp8 V layout transform idea)
+    perm = np.random.default_rng(0).permutation(S)
+    op = oracle.attention_f32(q, k[:, perm], v[:, perm])["O"]
+    assert np.max(np.abs(o - op)) < 2e-6
+    # one dominant key selects its V row
+    kd = k.copy()
+    kd[0, 5, 0, :] = 0
+    qd = q.copy()
+    qd[0, :, 0, :] = 0
+    qd[0, :, 0, 0] = 200.0
+    kd[0, :, 0, 0] = 0
+    kd[0, 5, 0, 0] = 1.0
+    od = oracle.attention_f32(qd, kd, v)["O"]
+    assert np.max(np.abs(od[0, :, 0, :] - v[0, 5, 0, :])) < 1e-5
+    # head / batch independence: changing head 1 leaves head 0 alone
+    v2 = v.copy()
+    v2[:, :, 1] += 1.0
+    o2 = oracle.attention_f32(q, k, v2)["O"]
+    assert np.array_equal(o2[:, :, 0], o[:, :, 0]) and not np.array_equal(o2[:, :, 1], o[:, :, 1])
+
+
+def test_integer_inputs_give_exact_scores():
+    # the reference's own exactness trick: integer-valued uniform [-8,8] inputs
+    # (include/utils/random.hpp:13-32, src/fmha/fmha_forward.cu:671-674)
+    rng = np.random.default_rng(22)
+    B, S, H, D = 1, 64, 2, 64
+    q = rng.integers(-8, 9, (B, S, H, D)).astype(np.float32)
+    k = rng.integers(-8, 9, (B, S, H, D)).astype(np.float32)
+    v = rng.integers(-8, 9, (B, S, H, D)).astype(np.float32)
+    r = oracle.attention_f32(q, k, v, alpha0=1.0, want_scores=True)
+    exact = np.einsum("bmhd,bnhd->bhmn", q.astype(np.int64), k.astype(np.int64))
+    assert np.array_equal(r["S"], exact.astype(np.float32))
+
+
+def test_subset_selection():
+    B, S, H, D = 2, 32, 3, 16
+    q, k, v = _rand((B, S, H, D), 23), _rand((B, S, H, D), 24), _rand((B, S, H, D), 25)
+    full = oracle.attention_f32(q, k, v)["O"]
+    sub = oracle.attention_f32(q, k, v, bh_pairs=[(1, 2), (0, 1)], row_start=3, row_step=5)["O"]
+    mask = np.zeros((B, S, H), bool)
+    mask[1, 3::5, 2] = True
+    mask[0, 3::5, 1] = True
+    assert np.array_equal(sub[mask], full[mask])
+    assert np.all(np.isnan(sub[~mask]))
+
+
+def test_gemm_oracle_exact_on_integers_and_layouts():
+    rng = np.random.default_rng(26)
+    M, N, K = 48, 40, 72
+    a = rng.integers(-8, 9, (M, K)).astype(np.float32)
+    b = rng.integers(-8, 9, (N, K)).astype(np.float32)
+    exact = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
+    assert np.array_equal(oracle.gemm_f32(a, b), exact)
+    assert np.array_equal(oracle.gemm_f32(a, np.ascontiguousarray(b.T), b_is_kn=True), exact)
+    rows = [5, 0, 47]
+    assert np.array_equal(oracle.gemm_f32(a, b, rows=rows), exact[rows])
+    # asymmetric problem: a transposed-operand mistake cannot pass
+    a2, b2 = _rand((M, K), 27), _rand((N, K), 28)
+    np.testing.assert_allclose(oracle.gemm_f32(a2, b2), a2.astype(np.float64) @ b2.astype(np.float64).T, atol=1e-4)
+
+
+def test_verify_tensor_semantics():
+    # include/utils/random.hpp:54-90: error iff NaN/Inf or (abs > 5e-3 AND rel > 1e-1)
+    ref = np.array([1.0, 1.0, 0.001, 0.001, 1.0, 0.0], np.float32)
+    x = np.array([1.004, 1.2, 0.0059, 0.007, np.nan, 0.004], np.float32)
+    #             ok(abs) bad    ok(abs<=5e-3) bad   bad     ok(abs)
+    ok, pct = oracle.verify_tensor(x, ref)
+    assert not ok and abs(pct - 100.0 * 3 / 6) < 1e-4
+    assert oracle.verify_tensor(x, ref, err_count_expected=50.0)[0]
+    assert oracle.verify_tensor(ref, ref)[0]
+    big = np.ones(2_000_000, np.float32)
+    one_bad = big.copy()
+    one_bad[7] = 2.0
+    assert oracle.verify_tensor(one_bad, big, 1e-4)[0]          # 5e-5 % <= 1e-4 %
+    one_bad[8] = 2.0
+    one_bad[9] = 2.0
+    assert not oracle.verify_tensor(one_bad, big, 1e-4)[0]      # 1.5e-4 % > 1e-4 %
+
+
+def test_e4m3_decode_table_closed_form_and_torch():
+    table = oracle.e4m3_decode_table()
+    assert table[0x7E] == 448.0 and table[0x01] == 2.0 ** -9 and table[0x08] == 2.0 ** -6
+    assert table[0x38] == 1.0 and table[0xB8] == -1.0 and np.isnan(table[0x7F]) and np.isnan(table[0xFF])
+    t = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    assert np.array_equal(np.nan_to_num(t, nan=12345.0), np.nan_to_num(table, nan=12345.0))
+
+
+def test_e4m3_encode_rne_saturating_all_midpoints():
+    table = oracle.e4m3_decode_table()
+    pos = table[:0x7F].astype(np.float64)
+    # exact values round-trip
+    assert np.array_equal(oracle.e4m3_encode(table[:0x7F]), np.arange(0x7F, dtype=np.uint8))
+    assert np.array_equal(oracle.e4m3_encode(-table[1:0x7F]), np.arange(1, 0x7F, dtype=np.uint8) | 0x80)
+    # midpoints go to the even code; just-above / just-below go to the nearer
+    mids = ((pos[:-1] + pos[1:]) / 2).astype(np.float32)
+    lo = np.arange(0x7E)
+    want = np.where(lo % 2 == 0, lo, lo + 1).astype(np.uint8)
+    assert np.array_equal(oracle.e4m3_encode(mids), want)
+    assert np.array_equal(oracle.e4m3_encode(np.nextafter(mids, np.float32(np.inf))), (lo + 1).astype(np.uint8))
+    assert np.array_equal(oracle.e4m3_encode(np.nextafter(mids, np.float32(-np.inf))), lo.astype(np.uint8))
+    # saturation and NaN
+    assert list(oracle.e4m3_encode(np.array([1e9, -1e9, 464.0, np.inf, np.nan], np.float32))) == [0x7E, 0xFE, 0x7E, 0x7E, 0x7F]
+    # agreement with torch's converter on the finite range (torch maps overflow to NaN, so clamp first)
+    x = (np.random.default_rng(29).standard_normal(200000) * 60).astype(np.float32).clip(-448, 448)
+    t = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(oracle.e4m3_encode(x), t)
+
+
+def test_fp16_roundtrip_exhaustive():
+    # numpy.float16 is IEEE binary16 with RNE; every code survives float32 and back, and float32
+    # midpoints between adjacent halves round to even
+    codes = np.arange(65536, dtype=np.uint16)
+    h = codes.view(np.float16)
+    back = h.astype(np.float32).astype(np.float16).view(np.uint16)
+    fin = ~np.isnan(h)
+    assert np.array_equal(back[fin], codes[fin])
+    pos = np.arange(0x0001, 0x7BFF, dtype=np.uint16)
+    a = pos.view(np.float16).astype(np.float32)
+    b = (pos + 1).astype(np.uint16).view(np.float16).astype(np.float32)
+    mid = ((a.astype(np.float64) + b.astype(np.float64)) / 2).astype(np.float32)
+    want = np.where(pos % 2 == 0, pos, pos + 1).astype(np.uint16)
+    assert np.array_equal(mid.astype(np.float16).view(np.uint16), want)
+
+
+def test_v_layouts():
+    v = np.arange(2 * 32 * 3 * 4, dtype=np.float32).reshape(2, 32, 3, 4)
+    vt = oracle.transpose_v_bdhs(v)
+    assert vt.shape == (2, 4, 3, 32) and vt[1, 2, 1, 7] == v[1, 7, 1, 2]
+    vp = oracle.permute_keys16(vt)
+    # dst[p + 2r + 8q] = src[p + 2q + 4r]
+    assert vp[0, 0, 0, 16 + 1 + 2 * 3 + 8 * 1] == vt[0, 0, 0, 16 + 1 + 2 * 1 + 4 * 3]
+    assert sorted(vp[0, 0, 0, :16]) == sorted(vt[0, 0, 0, :16])
+
+
+@pytest.mark.parametrize("bN", [16, 32, 64, 128])
+def test_online_tiled_softmax_equals_direct(bN):
+    # brute force: the kernel-side tiled algorithm (online_softmax.h:87-207) == direct softmax
+    S, D = 256, 64
+    q, k, v = _rand((S, D), 30), _rand((S, D), 31), _rand((S, D), 32)
+    scale = 1.0 / np.sqrt(D)
+    o, m, l = oracle.online_softmax_tiled(q, k, v, bN, scale * oracle.LOG2E, p_cast=None)
+    r = oracle.attention_f32(q[None, :, None], k[None, :, None], v[None, :, None], want_stats=True)
+    assert np.max(np.abs(o - r["O"][0, :, 0])) < 3e-6
+    # tap conventions: m in the log2 domain, l not reciprocal (fmha_forward.cu:655-676)
+    np.testing.assert_allclose(m / oracle.LOG2E, r["row_max"][0, 0], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(1.0 / l, r["inv_sum"][0, 0], rtol=1e-5)
+    # with P rounded to fp16 the error stays far inside the 2e-3 gate
+    o16, _, _ = oracle.online_softmax_tiled(q, k, v, bN, scale * oracle.LOG2E, p_cast="f16")
+    assert np.max(np.abs(o16 - r["O"][0, :, 0])) < 1e-3
