@@ -1,0 +1,152 @@
+// C-ABI of libcfk_fmha.so (declared in include/cfk_fmha.h): argument validation, kernel selection, launch.
+// Host-side counterpart of fmhaForwardDevice (src/fmha-pipeline/fmha_forward.cu:86-383): where the reference
+// builds TMA descriptors and picks a kernel by compile-time macros, this layer checks the run-time shape
+// against the tile plan and dispatches to a gfx950 instantiation.
+#include "../../include/cfk_fmha.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "fmha_common.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// Shape / enum checks shared by the plan query and the launch.  Fills `plan`.
+int check_fmha(const cfk_fmha_fwd_params *p, cfk::FmhaPlan *plan, bool need_pointers) {
+  if (!p) return fail(CFK_ERR_INVALID_ARG, "params is NULL");
+  if (p->dtype != CFK_FP16 && p->dtype != CFK_FP8_E4M3)
+    return fail(CFK_ERR_INVALID_ARG, "Unsupported type: %d (1 = fp16, 2 = fp8 e4m3)", p->dtype);
+  if (p->v_dtype != CFK_FP16 && p->v_dtype != CFK_FP8_E4M3)
+    return fail(CFK_ERR_INVALID_ARG, "Unsupported V type: %d", p->v_dtype);
+  if (p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_kv <= 0)
+    return fail(CFK_ERR_INVALID_ARG, "batch, heads, seqlen_q, seqlen_kv must be positive (got %d, %d, %d, %d)",
+                p->batch, p->heads, p->seqlen_q, p->seqlen_kv);
+  if (p->head_dim != 64 && p->head_dim != 128 && p->head_dim != 256)
+    return fail(CFK_ERR_UNSUPPORTED, "Unsupported head dim: %d", p->head_dim);
+  if (p->v_layout != CFK_V_BSHD && p->v_layout != CFK_V_BDHS)
+    return fail(CFK_ERR_INVALID_ARG, "unknown v_layout %d", p->v_layout);
+  if (p->dtype != p->v_dtype)
+    return fail(CFK_ERR_UNSUPPORTED, "hybrid precision (Q,K fp8 with fp16 P,V) is not built; v_dtype must equal dtype");
+  if (p->dtype == CFK_FP16 && p->v_layout != CFK_V_BSHD)
+    return fail(CFK_ERR_UNSUPPORTED, "pre-transposed V ([B,D,H,S]) is accepted for fp8 only");
+  if (!(p->softmax_scale > 0.f) || !std::isfinite(p->softmax_scale))
+    return fail(CFK_ERR_INVALID_ARG, "softmax_scale must be positive and finite");
+  if (p->dtype == CFK_FP8_E4M3) {
+    const float d[3] = {p->q_descale, p->k_descale, p->v_descale};
+    for (float x : d)
+      if (!(x > 0.f) || !std::isfinite(x)) return fail(CFK_ERR_INVALID_ARG, "fp8 descales must be positive and finite");
+  }
+  const long long bh = (long long)p->batch * p->heads;
+  if (bh > (1 << 24)) return fail(CFK_ERR_UNSUPPORTED, "batch*heads too large");
+  bool ok = p->dtype == CFK_FP16 ? cfk::plan_fmha_f16(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, plan)
+                                 : cfk::plan_fmha_fp8(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, p->v_layout, plan);
+  if (!ok) return fail(CFK_ERR_UNSUPPORTED, "no kernel for dtype %d head dim %d v_layout %d", p->dtype, p->head_dim, p->v_layout);
+  // The kernels carry no masks, exactly like the reference (no bounds handling: fmha_forward.cu:361-372).
+  if (p->seqlen_q % plan->block_m != 0)
+    return fail(CFK_ERR_UNSUPPORTED, "seqlen_q %d is not a multiple of the query tile %d", p->seqlen_q, plan->block_m);
+  if (p->seqlen_kv % plan->block_n != 0)
+    return fail(CFK_ERR_UNSUPPORTED, "seqlen_kv %d is not a multiple of the key tile %d", p->seqlen_kv, plan->block_n);
+  const long long elems = bh * (long long)(p->seqlen_q > p->seqlen_kv ? p->seqlen_q : p->seqlen_kv) * p->head_dim;
+  if (elems >= (1LL << 40)) return fail(CFK_ERR_UNSUPPORTED, "tensor too large");
+  if (need_pointers && (!p->q || !p->k || !p->v || !p->o))
+    return fail(CFK_ERR_INVALID_ARG, "q, k, v, o must be non-NULL device pointers");
+  return CFK_OK;
+}
+
+int check_device() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(CFK_ERR_NO_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+  static thread_local int checked_dev = -1;
+  if (checked_dev == dev) return CFK_OK;
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, dev);
+  if (e != hipSuccess) return fail(CFK_ERR_HIP, "hipGetDeviceProperties: %s", hipGetErrorString(e));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(CFK_ERR_NO_DEVICE, "device %d is %s; this library is built for gfx950 only", dev, prop.gcnArchName);
+  checked_dev = dev;
+  return CFK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int cfk_fmha_forward_plan(const cfk_fmha_fwd_params *params, int32_t *block_m, int32_t *block_n, int32_t *lds_bytes,
+                          int32_t *threads) {
+  cfk::FmhaPlan plan{};
+  int rc = check_fmha(params, &plan, false);
+  if (rc != CFK_OK) return rc;
+  if (block_m) *block_m = plan.block_m;
+  if (block_n) *block_n = plan.block_n;
+  if (lds_bytes) *lds_bytes = plan.lds_bytes;
+  if (threads) *threads = plan.threads;
+  return CFK_OK;
+}
+
+int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
+  cfk::FmhaPlan plan{};
+  int rc = check_fmha(p, &plan, true);
+  if (rc != CFK_OK) return rc;
+  rc = check_device();
+  if (rc != CFK_OK) return rc;
+  constexpr float kLog2e = 1.4426950408889634074f;  // fmha_forward.cu:452
+  cfk::FmhaArgs a{};
+  a.q = p->q;
+  a.k = p->k;
+  a.v = p->v;
+  a.o = p->o;
+  a.row_max = p->dbg_row_max;
+  a.row_sum = p->dbg_row_sum;
+  a.B = p->batch;
+  a.H = p->heads;
+  a.Sq = p->seqlen_q;
+  a.Skv = p->seqlen_kv;
+  a.v_layout = p->v_layout;
+  hipError_t e;
+  if (p->dtype == CFK_FP16) {
+    a.scale_log2 = p->softmax_scale * kLog2e;
+    a.out_scale = 1.0f;
+    e = cfk::launch_fmha_f16(a, p->head_dim, (hipStream_t)stream);
+  } else {
+    a.scale_log2 = p->softmax_scale * kLog2e * p->q_descale * p->k_descale;
+    a.out_scale = p->v_descale;
+    e = cfk::launch_fmha_fp8(a, p->head_dim, (hipStream_t)stream);
+  }
+  if (e != hipSuccess) return fail(CFK_ERR_HIP, "FMHA launch failed: %s", hipGetErrorString(e));
+  return CFK_OK;
+}
+
+int cfk_gemm_f16(int32_t M, int32_t N, int32_t K, const void *A, const void *B, void *C, int32_t layout, void *stream) {
+  if (M <= 0 || N <= 0 || K <= 0) return fail(CFK_ERR_INVALID_ARG, "M, N, K must be positive (got %d, %d, %d)", M, N, K);
+  if (!A || !B || !C) return fail(CFK_ERR_INVALID_ARG, "A, B, C must be non-NULL device pointers");
+  if (layout != CFK_GEMM_TN && layout != CFK_GEMM_NN) return fail(CFK_ERR_INVALID_ARG, "unknown GEMM layout %d", layout);
+  if (M % 256 || N % 256 || K % 64)
+    return fail(CFK_ERR_UNSUPPORTED, "M and N must be multiples of 256 and K of 64 (got %d, %d, %d)", M, N, K);
+  int rc = check_device();
+  if (rc != CFK_OK) return rc;
+  hipError_t e = cfk::launch_gemm_f16(M, N, K, A, B, C, layout, (hipStream_t)stream);
+  if (e == hipErrorNotSupported) return fail(CFK_ERR_UNSUPPORTED, "GEMM layout %d is not built", layout);
+  if (e != hipSuccess) return fail(CFK_ERR_HIP, "GEMM launch failed: %s", hipGetErrorString(e));
+  return CFK_OK;
+}
+
+const char *cfk_last_error(void) { return g_err; }
+
+const char *cfk_version(void) { return "cfk-mi355x 0.1 gfx950"; }
+
+}  // extern "C"

@@ -1,0 +1,180 @@
+"""ctypes binding of the C-ABI in ``include/cfk_fmha.h``.
+
+Mirrors the reference's host entry ``fmhaForwardDevice`` (src/fmha-pipeline/fmha_forward.cu:86-93): device
+pointers for Q/K/V/O in [B,S,H,D], sizes, softmax scale, precision.  torch is used only to own device memory
+and streams; all compute happens in ``libcfk_fmha.so``.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libcfk_fmha.so")
+_lib = None
+
+CFK_FP16 = 1
+CFK_FP8_E4M3 = 2
+CFK_V_BSHD = 0
+CFK_V_BDHS = 1
+CFK_GEMM_TN = 0
+CFK_GEMM_NN = 1
+
+
+class CfkError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"cfk error {code}: {msg}")
+        self.code = code
+
+
+class FmhaFwdParams(ctypes.Structure):
+    """``cfk_fmha_fwd_params`` (include/cfk_fmha.h)."""
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("v_dtype", ctypes.c_int32),
+        ("batch", ctypes.c_int32), ("heads", ctypes.c_int32),
+        ("seqlen_q", ctypes.c_int32), ("seqlen_kv", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32), ("v_layout", ctypes.c_int32),
+        ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p), ("o", ctypes.c_void_p),
+        ("softmax_scale", ctypes.c_float),
+        ("q_descale", ctypes.c_float), ("k_descale", ctypes.c_float), ("v_descale", ctypes.c_float),
+        ("dbg_row_max", ctypes.c_void_p), ("dbg_row_sum", ctypes.c_void_p),
+    ]
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def build(verbose: bool = False) -> str:
+    """Compile every HIP source for gfx950 (``make -C csrc``; always recompiles what changed)."""
+    cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-j8"]
+    res = subprocess.run(cmd, capture_output=not verbose, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("building libcfk_fmha.so failed:\n" + (res.stdout or "") + (res.stderr or ""))
+    return _LIB_PATH
+
+
+def lib():
+    """The loaded C-ABI library.  Raises if it has not been built -- there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build it first (python -c 'import __graft_entry__ as g; g.build()' "
+                f"or make -C {os.path.join(_HERE, 'csrc')}). There is no CPU fallback.")
+        l = ctypes.CDLL(_LIB_PATH)
+        l.cfk_fmha_forward.restype = ctypes.c_int
+        l.cfk_fmha_forward.argtypes = [ctypes.POINTER(FmhaFwdParams), ctypes.c_void_p]
+        l.cfk_fmha_forward_plan.restype = ctypes.c_int
+        l.cfk_fmha_forward_plan.argtypes = [ctypes.POINTER(FmhaFwdParams)] + [ctypes.POINTER(ctypes.c_int32)] * 4
+        l.cfk_gemm_f16.restype = ctypes.c_int
+        l.cfk_gemm_f16.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p] * 3 + [ctypes.c_int32, ctypes.c_void_p]
+        l.cfk_last_error.restype = ctypes.c_char_p
+        l.cfk_version.restype = ctypes.c_char_p
+        _lib = l
+    return _lib
+
+
+def last_error() -> str:
+    return lib().cfk_last_error().decode()
+
+
+def version() -> str:
+    return lib().cfk_version().decode()
+
+
+def _check(rc):
+    if rc != 0:
+        raise CfkError(rc, last_error())
+
+
+def make_params(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, q=0, k=0, v=0, o=0, softmax_scale=None,
+                q_descale=1.0, k_descale=1.0, v_descale=1.0, v_layout=CFK_V_BSHD, v_dtype=None,
+                dbg_row_max=0, dbg_row_sum=0) -> FmhaFwdParams:
+    p = FmhaFwdParams()
+    p.dtype = dtype
+    p.v_dtype = dtype if v_dtype is None else v_dtype
+    p.batch, p.heads, p.seqlen_q, p.seqlen_kv, p.head_dim = batch, heads, seqlen_q, seqlen_kv, head_dim
+    p.v_layout = v_layout
+    p.q, p.k, p.v, p.o = q or None, k or None, v or None, o or None
+    p.softmax_scale = (1.0 / math.sqrt(head_dim)) if softmax_scale is None else softmax_scale
+    p.q_descale, p.k_descale, p.v_descale = q_descale, k_descale, v_descale
+    p.dbg_row_max = dbg_row_max or None
+    p.dbg_row_sum = dbg_row_sum or None
+    return p
+
+
+def fmha_forward_plan(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, v_layout=CFK_V_BSHD, v_dtype=None):
+    """(block_m, block_n, lds_bytes, threads) the library picks; raises CfkError for unsupported shapes.  No GPU needed."""
+    p = make_params(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, v_layout=v_layout, v_dtype=v_dtype)
+    out = [ctypes.c_int32() for _ in range(4)]
+    _check(lib().cfk_fmha_forward_plan(ctypes.byref(p), *[ctypes.byref(x) for x in out]))
+    return tuple(x.value for x in out)
+
+
+def _stream_ptr(stream):
+    if stream is None:
+        import torch
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return ctypes.c_void_p(stream if isinstance(stream, int) else stream.cuda_stream)
+
+
+def fmha_forward(q, k, v, o=None, softmax_scale=None, q_descale=1.0, k_descale=1.0, v_descale=1.0,
+                 v_layout=CFK_V_BSHD, row_max=None, row_sum=None, stream=None):
+    """O = softmax(scale * Q K^T) V on device tensors in [B,S,H,D] (D contiguous).
+
+    q,k,v: torch CUDA tensors, float16, or float8_e4m3fn / uint8 holding e4m3 codes.  ``v`` is [B,D,H,S] when
+    ``v_layout == CFK_V_BDHS``.  Returns ``o`` (float16 [B,Sq,H,D]); launches asynchronously on ``stream``
+    (default: torch's current stream)."""
+    import torch
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise ValueError("q, k, v must be device tensors (there is no CPU path)")
+    if not (q.is_contiguous() and k.is_contiguous() and v.is_contiguous()):
+        raise ValueError("q, k, v must be contiguous [B,S,H,D]")
+    if q.dtype == torch.float16:
+        dtype = CFK_FP16
+    elif q.dtype in (torch.float8_e4m3fn, torch.uint8):
+        dtype = CFK_FP8_E4M3
+    else:
+        raise ValueError(f"unsupported dtype {q.dtype}")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k, v must share one dtype")
+    B, Sq, H, D = q.shape
+    Skv = k.shape[1]
+    if tuple(k.shape) != (B, Skv, H, D):
+        raise ValueError("k shape mismatch")
+    want_v = (B, Skv, H, D) if v_layout == CFK_V_BSHD else (B, D, H, Skv)
+    if tuple(v.shape) != want_v:
+        raise ValueError(f"v shape {tuple(v.shape)} does not match layout {v_layout}: expected {want_v}")
+    if o is None:
+        o = torch.empty((B, Sq, H, D), dtype=torch.float16, device=q.device)
+    elif o.dtype != torch.float16 or tuple(o.shape) != (B, Sq, H, D) or not o.is_contiguous() or not o.is_cuda:
+        raise ValueError("o must be a contiguous float16 device tensor [B,Sq,H,D]")
+    for t in (row_max, row_sum):
+        if t is not None and (t.dtype != torch.float32 or tuple(t.shape) != (B, H, Sq) or not t.is_contiguous()):
+            raise ValueError("row_max/row_sum must be contiguous float32 [B,H,Sq]")
+    p = make_params(dtype, B, H, Sq, Skv, D, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), softmax_scale,
+                    q_descale, k_descale, v_descale, v_layout,
+                    dbg_row_max=row_max.data_ptr() if row_max is not None else 0,
+                    dbg_row_sum=row_sum.data_ptr() if row_sum is not None else 0)
+    _check(lib().cfk_fmha_forward(ctypes.byref(p), _stream_ptr(stream)))
+    return o
+
+
+def gemm_f16(a, b, c=None, layout=CFK_GEMM_TN, stream=None):
+    """C[M,N] = A[M,K] . B  with B as [N,K] (TN, the reference's form) or [K,N] (NN); fp16 in, fp32 accumulate, fp16 out."""
+    import torch
+    if a.dtype != torch.float16 or b.dtype != torch.float16 or not (a.is_cuda and b.is_cuda):
+        raise ValueError("a, b must be float16 device tensors")
+    if not (a.is_contiguous() and b.is_contiguous()):
+        raise ValueError("a, b must be contiguous")
+    M, K = a.shape
+    N = b.shape[0] if layout == CFK_GEMM_TN else b.shape[1]
+    if tuple(b.shape) != ((N, K) if layout == CFK_GEMM_TN else (K, N)):
+        raise ValueError("b shape mismatch")
+    if c is None:
+        c = torch.empty((M, N), dtype=torch.float16, device=a.device)
+    _check(lib().cfk_gemm_f16(M, N, K, a.data_ptr(), b.data_ptr(), c.data_ptr(), layout, _stream_ptr(stream)))
+    return c

@@ -1,0 +1,108 @@
+/*
+ * cfk_fmha.h -- C-ABI of libcfk_fmha.so: fused multi-head-attention forward (fp16 and fp8 e4m3) and the
+ * dense fp16 GEMM example for AMD Instinct MI355X (gfx950).
+ *
+ * The reference repository (ColfaxResearch/cutlass-kernels) has no FFI: its hot path sits behind the C++
+ * template fmhaForwardDevice<PrecType, Gemm2Type, SoftType, OutputType, HEADDIM>
+ * (src/fmha-pipeline/fmha_forward.cu:86-93), called by its driver through fmhaForwardDeviceLoop
+ * (src/fmha-pipeline/fmha_forward.cu:387-419, call sites :578-592).  The entry points below carry that same
+ * contract over plain pointers and sizes so that a driver written against the reference's host function can
+ * call HIP where it called CUDA.
+ *
+ * All pointers are DEVICE pointers owned by the caller; nothing is allocated, freed or retained by the
+ * library; every call is asynchronous on `stream` (a hipStream_t passed as void*, NULL = default stream).
+ * Functions return CFK_OK (0) or a negative cfk_status; cfk_last_error() holds a message for the calling
+ * thread's last failure.  The library never calls exit() (the reference does, :758-760).
+ */
+#ifndef CFK_FMHA_H_
+#define CFK_FMHA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum cfk_status {
+  CFK_OK = 0,
+  CFK_ERR_INVALID_ARG = -1, /* null pointer, non-positive size, unknown enum value            */
+  CFK_ERR_UNSUPPORTED = -2, /* head dim / precision / layout / tile divisibility not supported */
+  CFK_ERR_HIP = -3,         /* a HIP runtime call failed (message names it)                    */
+  CFK_ERR_NO_DEVICE = -4    /* no gfx950 device is current                                     */
+} cfk_status;
+
+/* Operand precision; values mirror the driver flag --prec-type (src/fmha-pipeline/fmha_forward.cu:694,733). */
+typedef enum cfk_dtype { CFK_FP16 = 1, CFK_FP8_E4M3 = 2 } cfk_dtype;
+
+/* Layout of V in memory. */
+typedef enum cfk_v_layout {
+  CFK_V_BSHD = 0, /* [B, S_kv, H, D], D contiguous -- the reference's default (fmha_forward.cu:189-190)       */
+  CFK_V_BDHS = 1  /* [B, D, H, S_kv], S contiguous -- the reference's offline pre-transposed fp8 V (GEMM2FP8,
+                     fmha_forward.cu:231-232, 514-532); accepted for fp8 only                                   */
+} cfk_v_layout;
+
+/*
+ * Arguments of one forward call.  Replaces the argument list of fmhaForwardDevice
+ * (src/fmha-pipeline/fmha_forward.cu:88-93): SEQLEN, KEYLEN, NUMHEADS, BATCH, tensorQ/K/V, tensorS, tensorO,
+ * miOut, sPrimeOut, scale, stream; HEADDIM and the precisions are run-time fields here instead of template
+ * parameters.  The reference's `iterations` argument (a launch loop inside the entry) is the caller's loop here.
+ */
+typedef struct cfk_fmha_fwd_params {
+  int32_t dtype;     /* cfk_dtype of Q and K                                                                  */
+  int32_t v_dtype;   /* cfk_dtype of V (and of P): must equal dtype; CFK_FP16 with dtype = CFK_FP8_E4M3 is the
+                        reference's hybrid mode (fmha_forward.cu:446-450) and is reported CFK_ERR_UNSUPPORTED */
+  int32_t batch;     /* BATCH                                                                                 */
+  int32_t heads;     /* NUMHEADS                                                                              */
+  int32_t seqlen_q;  /* SEQLEN: multiple of 128                                                               */
+  int32_t seqlen_kv; /* KEYLEN: multiple of 128                                                               */
+  int32_t head_dim;  /* HEADDIM: 64, 128 or 256 (fmha_forward.cu:746-761)                                     */
+  int32_t v_layout;  /* cfk_v_layout                                                                          */
+  const void *q;     /* [B, S_q,  H, D] dtype, D contiguous (fmha_forward.cu:151-152)                         */
+  const void *k;     /* [B, S_kv, H, D] dtype               (fmha_forward.cu:162-163)                         */
+  const void *v;     /* v_layout, v_dtype                                                                     */
+  void *o;           /* [B, S_q, H, D] fp16, always (fmha_forward.cu:245-246, 471)                            */
+  float softmax_scale; /* natural-domain scale, normally 1/sqrt(D); the library multiplies by log2(e) itself.
+                          (The reference passes scale*log2e, fmha_forward.cu:452-454.)                        */
+  float q_descale;   /* fp8 per-tensor scales: real value = code value * descale.  1.0f reproduces the        */
+  float k_descale;   /* reference, which applies no scaling (fmha_forward.cu:498-500).  Ignored for fp16.     */
+  float v_descale;
+  float *dbg_row_max; /* optional tap, [B, H, S_q] fp32: running row max in the log2 domain (score*scale*log2e),
+                         the reference's miOut under COPYOUTMI (fmha_epilogue.h:7-46); NULL = off              */
+  float *dbg_row_sum; /* optional tap, [B, H, S_q] fp32: row sum of exp2(t - max), not its reciprocal, the
+                         reference's sPrimeOut (fmha_forward.cu:668-672); NULL = off                           */
+} cfk_fmha_fwd_params;
+
+/* FMHA forward: O = softmax(softmax_scale * Q K^T) V per (batch, head); no mask, no dropout.
+ * Replaces fmhaForwardDevice (src/fmha-pipeline/fmha_forward.cu:86-383), one launch per call. */
+int cfk_fmha_forward(const cfk_fmha_fwd_params *params, void *stream);
+
+/* Bytes of LDS and the tile shape the library would pick for `params` (query rows per workgroup, keys per
+ * tile); the reference fixes these at compile time (src/fmha-pipeline/shared_storage.h:4-22).  Any of the
+ * out-pointers may be NULL.  Does not touch the GPU. */
+int cfk_fmha_forward_plan(const cfk_fmha_fwd_params *params, int32_t *block_m, int32_t *block_n,
+                          int32_t *lds_bytes, int32_t *threads);
+
+/* GEMM layouts for cfk_gemm_f16. */
+typedef enum cfk_gemm_layout {
+  CFK_GEMM_TN = 0, /* A: M x K (K contiguous), B: N x K (K contiguous) -- the reference's form
+                      (src/cute-gemm-tma-gma/gemm.cu:362-380)                                                  */
+  CFK_GEMM_NN = 1  /* A: M x K (K contiguous), B: K x N (N contiguous) -- the literal C = A.B                  */
+} cfk_gemm_layout;
+
+/* Dense GEMM C = A.B (fp16 operands, fp32 accumulate, fp16 C row-major M x N, N contiguous).
+ * Replaces gemm(...) of the CuTe example (src/cute-gemm-tma-gma/gemm.cu:336-463) with alpha = 1, beta = 0.
+ * M, N multiples of 256; K a multiple of 64. */
+int cfk_gemm_f16(int32_t M, int32_t N, int32_t K, const void *A, const void *B, void *C, int32_t layout,
+                 void *stream);
+
+/* Message for the calling thread's most recent non-zero return ("" if none). */
+const char *cfk_last_error(void);
+
+/* "cfk-mi355x <version> gfx950" */
+const char *cfk_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CFK_FMHA_H_ */

@@ -1,0 +1,74 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol the header declares, validates
+arguments the way the reference driver's error paths do, and the plan query works without a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from _util import ROOT, pkg
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "cfk_fmha.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cfk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_functions()
+    assert {"cfk_fmha_forward", "cfk_fmha_forward_plan", "cfk_gemm_f16", "cfk_last_error", "cfk_version"} <= set(names)
+    lib = ctypes.CDLL(pkg.lib_path())
+    for n in names:
+        assert getattr(lib, n) is not None, n
+
+
+def test_params_struct_matches_header_layout():
+    # 8 int32, 4 pointers, 4 floats, 2 pointers on LP64
+    assert ctypes.sizeof(pkg.fmha.FmhaFwdParams) == 8 * 4 + 4 * 8 + 4 * 4 + 2 * 8
+    assert pkg.fmha.FmhaFwdParams.q.offset == 32 and pkg.fmha.FmhaFwdParams.softmax_scale.offset == 64
+    assert pkg.fmha.FmhaFwdParams.dbg_row_max.offset == 80
+
+
+def test_version_and_plan_without_gpu():
+    assert "gfx950" in pkg.version()
+    bm, bn, lds, threads = pkg.fmha_forward_plan(pkg.CFK_FP16, 8, 16, 2048, 2048, 128)
+    assert 2048 % bm == 0 and 2048 % bn == 0 and 0 < lds <= 160 * 1024 and threads % 64 == 0
+    for d in (64, 128, 256):
+        pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, d)
+
+
+def test_error_paths_mirror_reference_driver():
+    # unsupported head dim (fmha_forward.cu:758-760) and precision (:788-790) -> error codes, never exit()
+    with pytest.raises(pkg.CfkError) as e:
+        pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, 96)
+    assert e.value.code == -2 and "Unsupported head dim: 96" in str(e.value)
+    with pytest.raises(pkg.CfkError) as e:
+        pkg.fmha_forward_plan(3, 1, 1, 512, 512, 64)
+    assert e.value.code == -1 and "Unsupported type: 3" in str(e.value)
+    with pytest.raises(pkg.CfkError) as e:
+        pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 500, 512, 64)  # no masks: tiles must divide S
+    assert e.value.code == -2
+    with pytest.raises(pkg.CfkError) as e:
+        pkg.fmha_forward_plan(pkg.CFK_FP16, 0, 1, 512, 512, 64)
+    assert e.value.code == -1
+    with pytest.raises(pkg.CfkError):
+        pkg.fmha_forward_plan(pkg.CFK_FP8_E4M3, 1, 1, 512, 512, 64, v_dtype=pkg.CFK_FP16)  # hybrid mode not built
+    with pytest.raises(pkg.CfkError):
+        pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, 64, v_layout=1)
+    # null params / null pointers
+    lib = pkg.lib()
+    assert lib.cfk_fmha_forward(None, None) == -1
+    p = pkg.fmha.make_params(pkg.CFK_FP16, 1, 1, 512, 512, 64)
+    assert lib.cfk_fmha_forward(ctypes.byref(p), None) == -1 and "non-NULL" in pkg.last_error()
+    p = pkg.fmha.make_params(pkg.CFK_FP16, 1, 1, 512, 512, 64, softmax_scale=-1.0)
+    assert lib.cfk_fmha_forward_plan(ctypes.byref(p), None, None, None, None) == -1
+    assert lib.cfk_gemm_f16(100, 256, 64, None, None, None, 0, None) == -1
+    assert lib.cfk_gemm_f16(100, 256, 64, 1, 1, 1, 0, None) == -2
+
+
+def test_python_binding_refuses_cpu_tensors():
+    import torch
+    x = torch.zeros((1, 128, 1, 64), dtype=torch.float16)
+    with pytest.raises(ValueError):
+        pkg.fmha_forward(x, x, x)

@@ -1,0 +1,131 @@
+"""GPU parity of the fp16 FMHA forward (through the C-ABI) against the CPU oracle on the same seeded inputs.
+Gate: max-abs error <= 2e-3 against the fp32 host reference attention, plus the reference's own error-percentage
+criterion (include/utils/random.hpp:54-90, thresholds src/fmha-pipeline/fmha_forward.cu:638-639)."""
+import numpy as np
+import pytest
+
+import oracle
+from _util import ERRPCT_FP16, TOL_FP16, max_abs, pkg, subset_pairs, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(q, k, v, **kw):
+    import torch
+    q16, k16, v16 = (x.astype(np.float16) for x in (q, k, v))
+    o = pkg.fmha_forward(to_dev(q16), to_dev(k16), to_dev(v16), **kw)
+    torch.cuda.synchronize()
+    return o.float().cpu().numpy(), (q16.astype(np.float32), k16.astype(np.float32), v16.astype(np.float32))
+
+
+def _check_full(B, S, H, D, kind="gaussian", seqlen_kv=None, scale=None):
+    q, k, v = pkg.testbed.qkv(B, S, H, D, kind=kind, seqlen_kv=seqlen_kv)
+    if kind != "gaussian":
+        q, k = q / 8, k / 8  # keep scores moderate
+    got, (qf, kf, vf) = _run(q, k, v, softmax_scale=scale)
+    ref = oracle.attention_f32(qf, kf, vf, alpha0=scale)["O"]
+    err = max_abs(got, ref)
+    ok, pct = oracle.verify_tensor(got, ref, ERRPCT_FP16)
+    print(f"fp16 B={B} S={S}/{seqlen_kv or S} H={H} D={D} {kind}: max-abs {err:.3e}, error% {pct:.2e}")
+    assert err <= TOL_FP16, err
+    assert ok, pct
+
+
+def test_config1_full_check():
+    # BASELINE config 1: B=1 H=8 S=512 D=64, scale 1/sqrt(64), full CPU check
+    _check_full(1, 512, 8, 64, scale=1.0 / 8.0)
+
+
+@pytest.mark.parametrize("B,S,H,D", [(2, 256, 3, 128), (1, 384, 2, 256), (3, 128, 5, 64), (1, 1024, 1, 128)])
+def test_head_dims_and_ragged_grids(B, S, H, D):
+    _check_full(B, S, H, D)
+
+
+def test_rectangular_q_kv():
+    _check_full(1, 256, 2, 128, seqlen_kv=640)
+    _check_full(2, 512, 2, 64, seqlen_kv=128)
+
+
+def test_integer_valued_inputs():
+    _check_full(1, 256, 2, 64, kind="uniform_int")
+
+
+def test_nondefault_scale():
+    _check_full(1, 256, 2, 128, scale=0.05)
+
+
+def test_row_max_and_row_sum_taps():
+    # the reference's max-check / sum-check (fmha_forward.cu:655-676): kernel max is in the log2 domain,
+    # kernel sum is not reciprocal
+    import torch
+    B, S, H, D = 2, 256, 2, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    rm = torch.full((B, H, S), -1.0, dtype=torch.float32, device="cuda:0")
+    rs = torch.full((B, H, S), -1.0, dtype=torch.float32, device="cuda:0")
+    got, (qf, kf, vf) = _run(q, k, v, row_max=rm, row_sum=rs)
+    r = oracle.attention_f32(qf, kf, vf, want_stats=True)
+    assert max_abs(got, r["O"]) <= TOL_FP16
+    mi = rm.cpu().numpy() / oracle.LOG2E
+    assert oracle.verify_tensor(mi, r["row_max"])[0]
+    assert oracle.verify_tensor(1.0 / rs.cpu().numpy(), r["inv_sum"])[0]
+    np.testing.assert_allclose(mi, r["row_max"], rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(1.0 / rs.cpu().numpy(), r["inv_sum"], rtol=1e-4)
+
+
+def test_kernel_matches_tiled_emulation_closely():
+    # against the numpy emulation of the kernel-side algorithm (P rounded to fp16 per tile) the difference is
+    # rounding noise of the fp16 output only
+    B, S, H, D = 1, 256, 1, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    got, (qf, kf, vf) = _run(q, k, v)
+    bn = pkg.fmha_forward_plan(pkg.CFK_FP16, B, H, S, S, D)[1]
+    emu, _, _ = oracle.online_softmax_tiled(qf[0, :, 0], kf[0, :, 0], vf[0, :, 0], bn, oracle.LOG2E / np.sqrt(D))
+    assert max_abs(got[0, :, 0], emu) <= 6e-4
+
+
+def test_invariants_on_device():
+    import torch
+    B, S, H, D = 1, 512, 4, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    base, _ = _run(q, k, v)
+    # V = 1 -> O = 1 (rows of P sum to one)
+    ones, _ = _run(q, k, np.ones_like(v))
+    assert max_abs(ones, 1.0) <= 1e-3
+    # a common permutation of the keys changes nothing beyond rounding
+    perm = np.random.default_rng(5).permutation(S)
+    permd, _ = _run(q, k[:, perm], v[:, perm])
+    assert max_abs(base, permd) <= 1e-3
+    # Q = 0 -> mean of V
+    zero, (_, _, vf) = _run(np.zeros_like(q), k, v)
+    assert max_abs(zero, np.broadcast_to(vf.mean(axis=1, keepdims=True), vf.shape)) <= 1e-3
+    # output buffer is fully overwritten (the driver pre-fills O with -1, fmha_forward.cu:501-502)
+    o = torch.full((B, S, H, D), -1.0, dtype=torch.float16, device="cuda:0")
+    pkg.fmha_forward(to_dev(q.astype(np.float16)), to_dev(k.astype(np.float16)), to_dev(v.astype(np.float16)), o=o)
+    torch.cuda.synchronize()
+    assert max_abs(o.float().cpu().numpy(), base) == 0.0
+
+
+def _subset_check(B, S, H, D):
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    got, (qf, kf, vf) = _run(q, k, v)
+    pairs = subset_pairs(B, H)
+    ref = oracle.attention_f32(qf, kf, vf, bh_pairs=pairs)["O"]
+    all_pairs = [(b, h) for b in range(B) for h in range(H)]
+    oracle.attention_f32(qf, kf, vf, bh_pairs=all_pairs, row_start=17, row_step=61, out=ref)
+    sel = ~np.isnan(ref)
+    assert sel.sum() >= len(pairs) * S * D
+    err = max_abs(got[sel], ref[sel])
+    ok, pct = oracle.verify_tensor(got[sel], ref[sel], ERRPCT_FP16)
+    print(f"fp16 B={B} S={S} H={H} D={D}: checked {sel.sum()} elements, max-abs {err:.3e}, error% {pct:.2e}")
+    assert err <= TOL_FP16 and ok
+    assert not np.any(np.isnan(got)) and float(np.abs(got).max()) < 10.0
+
+
+def test_config2_headline_shape_subset_check():
+    # BASELINE config 2: B=8 H=16 S=2048 D=128; four full (b,h) slices + every 61st row of every head
+    _subset_check(8, 2048, 16, 128)
+
+
+def test_config3_long_sequence_large_head_subset_check():
+    # BASELINE config 3: B=2 H=8 S=8192 D=256
+    _subset_check(2, 8192, 8, 256)
