@@ -1,0 +1,184 @@
+#!/usr/bin/env python3
+"""FMHA-forward benchmark on one MI355X: prints ONE JSON line.
+
+Headline workload (BASELINE config 2): fp16, B=8 H=16 S=2048 D=128, non-causal, Q/K/V iid N(0,1) synthetic, fp32
+softmax/accumulate, fp16 output.  A "step" is one forward call over the whole batch through the C-ABI
+(``cfk_fmha_forward``), inputs resident in HBM.  FLOP = 4*B*H*Sq*Skv*D per step
+(src/fmha-pipeline/fmha_forward.cu:572-573); timing protocol = the reference's: warm-up launches, then the mean of
+K back-to-back launches between events (fmha_forward.cu:578-593).
+
+Also reported in the same line: ``roofline`` (MFMA-bound; achieved TFLOP/s over the measured mean launch duration
+against the published dense peak), ``cpu_baseline`` (the CPU oracle -- a restatement of the reference's host
+reference attention -- timed on this host's cores on a bounded sample of the same workload), and ``secondary``
+(the other single-GPU workloads: fp8 e4m3 config 4, the long-sequence config 3, the GEMM example).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f16": 2500.0, "f8": 5000.0}   # MI355X published dense MFMA peaks
+
+WORKLOADS = {
+    "cfg1": dict(kind="fmha", dtype="f16", B=1, H=8, S=512, D=64, scale=0.125),
+    "cfg2": dict(kind="fmha", dtype="f16", B=8, H=16, S=2048, D=128, scale=None),
+    "cfg3": dict(kind="fmha", dtype="f16", B=2, H=8, S=8192, D=256, scale=None),
+    "cfg4": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None),
+    "cfg5": dict(kind="gemm", dtype="f16", M=8192, N=8192, K=8192),
+}
+NAMES = {
+    "cfg1": "fmha_fwd fp16 B=1 H=8 S=512 D=64 non-causal",
+    "cfg2": "fmha_fwd fp16 B=8 H=16 S=2048 D=128 non-causal",
+    "cfg3": "fmha_fwd fp16 B=2 H=8 S=8192 D=256 non-causal",
+    "cfg4": "fmha_fwd fp8-e4m3 B=4 H=16 S=4096 D=128 non-causal, per-tensor amax scales, V [B,S,H,D]",
+    "cfg5": "gemm fp16 M=N=K=8192 TN fp32-accumulate",
+}
+
+
+def _time_launches(fn, steps, warmup):
+    """Mean launch duration in ms: `warmup` untimed calls, then exactly `steps` back-to-back calls between two
+    events recorded on the stream the kernels are launched on (torch's current stream)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return start.elapsed_time(stop) / steps, wall_ms / steps
+
+
+def _make_fmha(pkg, w, seed=3080):
+    import torch
+    dev = torch.device("cuda:0")
+    B, H, S, D = w["B"], w["H"], w["S"], w["D"]
+    gens = [torch.Generator(device=dev).manual_seed(seed + i) for i in (1, 2, 3)]
+    q, k, v = (torch.randn((B, S, H, D), generator=g, device=dev, dtype=torch.float32) for g in gens)
+    kw = dict(softmax_scale=w["scale"])
+    if w["dtype"] == "f16":
+        q, k, v = q.half(), k.half(), v.half()
+    else:
+        def quant(x):
+            s = float(x.abs().max()) / 448.0
+            return (x / s).clamp(-448, 448).to(torch.float8_e4m3fn), s
+        (q, qs), (k, ks), (v, vs) = quant(q), quant(k), quant(v)
+        kw.update(q_descale=qs, k_descale=ks, v_descale=vs)
+    o = torch.empty((B, S, H, D), dtype=torch.float16, device=dev)
+    flop = pkg.testbed.fmha_flops(B, H, S, S, D)
+    return (lambda: pkg.fmha_forward(q, k, v, o=o, **kw)), flop, (q, k, v, o, kw)
+
+
+def _make_gemm(pkg, w, seed=3080):
+    import torch
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(seed)
+    a = (torch.rand((w["M"], w["K"]), generator=g, device=dev) * 2 - 1).half()
+    b = (torch.rand((w["N"], w["K"]), generator=g, device=dev) * 2 - 1).half()
+    c = torch.empty((w["M"], w["N"]), dtype=torch.float16, device=dev)
+    return (lambda: pkg.gemm_f16(a, b, c=c)), 2.0 * w["M"] * w["N"] * w["K"], (a, b, c)
+
+
+def run_workload(pkg, name, steps, warmup):
+    w = WORKLOADS[name]
+    fn, flop, keep = (_make_fmha if w["kind"] == "fmha" else _make_gemm)(pkg, w)
+    ms, wall_ms = _time_launches(fn, steps, warmup)
+    tflops = flop / (ms * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[w["dtype"]]
+    return dict(workload=NAMES[name], ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, flop_per_step=flop,
+                dtype=w["dtype"], frac_of_peak=tflops / peak, peak_tflops=peak), keep
+
+
+def cpu_baseline(pkg, w, budget_s=12.0):
+    """Time the CPU oracle (restatement of TestAttention::compute, include/utils/fmha_cutlass.hpp:154-317) on whole
+    (batch, head) problems of the headline workload until ~budget_s of CPU work is done."""
+    import numpy as np
+    import oracle
+    B, H, S, D = 1, 2, w["S"], w["D"]
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    q, k, v = (x.astype(np.float16).astype(np.float32) for x in (q, k, v))
+    oracle.attention_f32(q, k, v, bh_pairs=[(0, 0)], row_start=0, row_step=64)  # warm-up (threads, pages)
+    heads = 0
+    t0 = time.perf_counter()
+    while True:
+        oracle.attention_f32(q, k, v, bh_pairs=[(0, heads % H)])
+        heads += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or heads >= 64:
+            break
+    flop = 4.0 * heads * S * S * D
+    return dict(value=flop / dt / 1e12, unit="TFLOP/s", cores=oracle.num_threads(), kind="port",
+                sample=f"{heads} whole (batch, head) problems of S={S} D={D} (fp32 host reference attention, "
+                       f"OpenMP), {dt:.1f} s of CPU time")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)     # reference default --iterations=20
+    ap.add_argument("--warmup", type=int, default=10)    # reference: 10 warm-up launches
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-secondary", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build is single-GPU (one MI355X); --gpus must be 1. "
+                 "Batch x heads shard without communication, see DESIGN.md.")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    import __graft_entry__ as entry
+    pkg = entry.load_package()
+    pkg.lib()  # fail loudly if the HIP library is missing
+
+    main_res, keep = run_workload(pkg, args.workload, args.steps, args.warmup)
+    del keep
+    torch.cuda.empty_cache()
+    secondary = []
+    if not args.no_secondary:
+        for name in sorted(WORKLOADS):
+            if name == args.workload or name == "cfg1":
+                continue
+            try:
+                r, keep = run_workload(pkg, name, args.steps, args.warmup)
+                del keep
+                torch.cuda.empty_cache()
+                secondary.append({k: r[k] for k in ("workload", "ms_per_step", "tflops", "dtype", "frac_of_peak")})
+            except pkg.CfkError as e:
+                secondary.append({"workload": NAMES[name], "error": str(e)})
+    w = WORKLOADS[args.workload]
+    out = {
+        "metric": "fmha_fwd_tflops",
+        "value": main_res["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": w["dtype"],
+        "data": "synthetic",
+        "config": {"workload": main_res["workload"], "flop_per_step": main_res["flop_per_step"],
+                   "layout": "[B,S,H,D]", "seeds": [3081, 3082, 3083]},
+        "roofline": {"bound": "mfma", "achieved": main_res["tflops"], "peak": main_res["peak_tflops"],
+                     "unit": "TFLOP/s", "frac": main_res["frac_of_peak"], "traffic": None},
+        "secondary": secondary,
+    }
+    if not args.no_cpu_baseline and w["kind"] == "fmha":
+        out["cpu_baseline"] = cpu_baseline(pkg, w)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
