@@ -62,6 +62,9 @@ int check_fmha(const cfk_fmha_fwd_params *p, cfk::FmhaPlan *plan, bool need_poin
     return fail(CFK_ERR_UNSUPPORTED, "seqlen_kv %d is not a multiple of the key tile %d", p->seqlen_kv, plan->block_n);
   const long long elems = bh * (long long)(p->seqlen_q > p->seqlen_kv ? p->seqlen_q : p->seqlen_kv) * p->head_dim;
   if (elems >= (1LL << 40)) return fail(CFK_ERR_UNSUPPORTED, "tensor too large");
+  // the kernels address one batch slice with 32-bit byte offsets
+  if ((long long)(p->seqlen_q > p->seqlen_kv ? p->seqlen_q : p->seqlen_kv) * p->heads * p->head_dim * 2 >= (1LL << 31))
+    return fail(CFK_ERR_UNSUPPORTED, "seqlen * heads * head_dim * 2 bytes must stay below 2 GiB per batch entry");
   if (need_pointers && (!p->q || !p->k || !p->v || !p->o))
     return fail(CFK_ERR_INVALID_ARG, "q, k, v, o must be non-NULL device pointers");
   return CFK_OK;
