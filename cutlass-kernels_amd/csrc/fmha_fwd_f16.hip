@@ -28,6 +28,7 @@
 //  * Workgroup ids are remapped so the query blocks of one head share an XCD's L2.
 #include <cstdlib>
 #include <type_traits>
+#include <utility>
 
 #include "fmha_common.h"
 
@@ -41,6 +42,15 @@ typedef short short4v __attribute__((ext_vector_type(4)));
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T *)(p))
 #define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+
+// Asynchronous 16 B/lane global -> LDS copy: lane l writes LDS bytes [lds_addr + 16 l, +16) with the 16 bytes at
+// its own global address.  Issued through inline asm on purpose: the compiler then does not track the copy, so it
+// does not drain vmcnt before every later LDS read, and the copies of one pipeline step stay in flight until
+// the explicit wait_lds_dma() in front of the step's closing barrier.  lds_addr must be wave-uniform.
+__device__ __forceinline__ void lds_dma16(const void *gptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void wait_lds_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 template <int D_, int BN_, int NQ_, int NWAVES_, int WPE_ = 1>
 struct F16Cfg {
@@ -114,12 +124,11 @@ fmha_fwd_f16_kernel(const FmhaArgs a) {
     goff_k[i] = (uint32_t)row * ld_bytes + (uint32_t)((cp ^ swz_k<D>(row)) * 16);
     goff_v[i] = (uint32_t)row * ld_bytes + (uint32_t)((cp ^ swz_v<D>(row)) * 16);
   }
+  const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
   auto load_tile = [&](const char *gbase, const uint32_t (&goff)[C::IPW], int jt, int lds_off) {
     const char *gt = gbase + (size_t)jt * tile_stride;
 #pragma unroll
-    for (int i = 0; i < C::IPW; ++i)
-      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(gt + goff[i]),
-                                       LDS_PTR(void, smem + lds_off + (i * C::NWAVES + wave) * 1024), 16, 0, 0);
+    for (int i = 0; i < C::IPW; ++i) lds_dma16(gt + goff[i], lds_base + lds_off + (i * C::NWAVES + wave) * 1024);
   };
   constexpr int K_ST0 = 0, V_ST0 = 2 * C::TILE_BYTES;
 
@@ -260,7 +269,8 @@ fmha_fwd_f16_kernel(const FmhaArgs a) {
     softmax_exp(s_cur, pb);
     pv(V_ST0 + P * C::TILE_BYTES, pb);
     if (HAS_NEXT) row_max_and_rescale(s_nxt);
-    __syncthreads();  // waits for this wave's copies (vmcnt) and LDS reads, then the workgroup barrier
+    wait_lds_dma();   // this wave's copies have landed ...
+    __syncthreads();  // ... and so have everybody else's; all reads of the stages about to be refilled are done
   };
 
   // ---- prologue: K_0, V_0, K_1 in flight; S_0 and its row max
@@ -268,6 +278,7 @@ fmha_fwd_f16_kernel(const FmhaArgs a) {
   load_tile(Kp, goff_k, 0, K_ST0);
   load_tile(Vp, goff_v, 0, V_ST0);
   load_tile(Kp, goff_k, n_tiles > 1 ? 1 : 0, K_ST0 + C::TILE_BYTES);
+  wait_lds_dma();
   __syncthreads();
   qk(K_ST0, s_a);
   row_max_and_rescale(s_a);
@@ -325,25 +336,30 @@ hipError_t launch_cfg(const FmhaArgs &a, hipStream_t s) {
   return hipGetLastError();
 }
 
-using Cfg64 = F16Cfg<64, 64, 1, 4, 2>;
-using Cfg128 = F16Cfg<128, 64, 1, 4, 2>;
-using Cfg256 = F16Cfg<256, 64, 1, 4, 1>;
-// experimental tile shapes for D = 128, selected with CFK_FMHA_VARIANT (tuning aid; the reference selects
-// its tile shape with -DQBLKSIZE/-DKBLKSIZE at compile time, src/fmha-pipeline/shared_storage.h:4-15)
-using Cfg128v1 = F16Cfg<128, 64, 1, 8, 2>;
-using Cfg128v2 = F16Cfg<128, 64, 2, 4, 1>;
-using Cfg128v3 = F16Cfg<128, 32, 2, 4, 1>;
-using Cfg128v4 = F16Cfg<128, 32, 1, 8, 2>;
-using Cfg128v5 = F16Cfg<128, 128, 1, 4, 1>;
-using Cfg128v6 = F16Cfg<128, 64, 1, 4, 1>;
-using Cfg128v7 = F16Cfg<128, 32, 1, 4, 2>;
+// Tile shapes.  "small" = 4 waves x 32 query rows (two workgroups share a CU), "large" = 8 waves x 32 rows (one
+// workgroup per CU, half the K/V traffic per query row); both run two waves per SIMD.
+using Cfg64S = F16Cfg<64, 64, 1, 4, 2>;
+using Cfg64L = F16Cfg<64, 64, 1, 8, 2>;
+using Cfg128S = F16Cfg<128, 64, 1, 4, 2>;
+using Cfg128L = F16Cfg<128, 64, 1, 8, 2>;
+using Cfg256S = F16Cfg<256, 32, 1, 4, 1>;   // one wave per SIMD: Q (64) + O (128) registers alone fill half the file
 
-int variant() {
-  static int v = [] {
-    const char *e = getenv("CFK_FMHA_VARIANT");
-    return e ? atoi(e) : 0;
+enum class Shape { S, L };
+
+// The reference fixes its tile shape at compile time (-DQBLKSIZE/-DKBLKSIZE, src/fmha-pipeline/shared_storage.h:4-15);
+// here it is picked per call: the large tile needs seqlen_q % 256 == 0 and enough workgroups to fill 256 CUs twice.
+// CFK_FMHA_TILE=small|large overrides the choice (tuning aid; ignored when the shape does not divide).
+Shape pick_shape(int head_dim, int sq, int bh) {
+  static const int forced = [] {
+    const char *e = getenv("CFK_FMHA_TILE");
+    if (!e) return -1;
+    return e[0] == 's' ? 0 : e[0] == 'l' ? 1 : -1;
   }();
-  return v;
+  if (head_dim == 256) return Shape::S;
+  const bool large_ok = sq % 256 == 0;
+  if (forced == 0 || !large_ok) return Shape::S;
+  if (forced == 1) return Shape::L;
+  return (long long)bh * (sq / 256) >= 512 ? Shape::L : Shape::S;
 }
 
 template <class C>
@@ -355,45 +371,29 @@ void fill_plan(int sq, int bh, FmhaPlan *p) {
   p->grid = bh * (sq / C::BM);
 }
 
-}  // namespace
-
-bool plan_fmha_f16(int head_dim, int sq, int skv, int bh, FmhaPlan *p) {
-  (void)skv;
+// calls f.template operator()<Cfg>() for the configuration chosen for this problem
+template <class F>
+bool dispatch(int head_dim, int sq, int bh, F &&f) {
+  const Shape sh = pick_shape(head_dim, sq, bh);
   switch (head_dim) {
-    case 64: fill_plan<Cfg64>(sq, bh, p); return true;
-    case 128:
-      switch (variant()) {
-        case 1: fill_plan<Cfg128v1>(sq, bh, p); return true;
-        case 2: fill_plan<Cfg128v2>(sq, bh, p); return true;
-        case 3: fill_plan<Cfg128v3>(sq, bh, p); return true;
-        case 4: fill_plan<Cfg128v4>(sq, bh, p); return true;
-        case 5: fill_plan<Cfg128v5>(sq, bh, p); return true;
-        case 6: fill_plan<Cfg128v6>(sq, bh, p); return true;
-        case 7: fill_plan<Cfg128v7>(sq, bh, p); return true;
-        default: fill_plan<Cfg128>(sq, bh, p); return true;
-      }
-    case 256: fill_plan<Cfg256>(sq, bh, p); return true;
+    case 64: sh == Shape::L ? f(Cfg64L{}) : f(Cfg64S{}); return true;
+    case 128: sh == Shape::L ? f(Cfg128L{}) : f(Cfg128S{}); return true;
+    case 256: f(Cfg256S{}); return true;
     default: return false;
   }
 }
 
+}  // namespace
+
+bool plan_fmha_f16(int head_dim, int sq, int skv, int bh, FmhaPlan *p) {
+  (void)skv;
+  return dispatch(head_dim, sq, bh, [&](auto cfg) { fill_plan<decltype(cfg)>(sq, bh, p); });
+}
+
 hipError_t launch_fmha_f16(const FmhaArgs &a, int head_dim, hipStream_t s) {
-  switch (head_dim) {
-    case 64: return launch_cfg<Cfg64>(a, s);
-    case 128:
-      switch (variant()) {
-        case 1: return launch_cfg<Cfg128v1>(a, s);
-        case 2: return launch_cfg<Cfg128v2>(a, s);
-        case 3: return launch_cfg<Cfg128v3>(a, s);
-        case 4: return launch_cfg<Cfg128v4>(a, s);
-        case 5: return launch_cfg<Cfg128v5>(a, s);
-        case 6: return launch_cfg<Cfg128v6>(a, s);
-        case 7: return launch_cfg<Cfg128v7>(a, s);
-        default: return launch_cfg<Cfg128>(a, s);
-      }
-    case 256: return launch_cfg<Cfg256>(a, s);
-    default: return hipErrorInvalidValue;
-  }
+  hipError_t e = hipErrorInvalidValue;
+  dispatch(head_dim, a.Sq, a.B * a.H, [&](auto cfg) { e = launch_cfg<decltype(cfg)>(a, s); });
+  return e;
 }
 
 }  // namespace cfk
