@@ -50,6 +50,21 @@ def test_integer_valued_inputs():
     _check_full(1, 256, 2, 64, kind="uniform_int")
 
 
+def test_exact_arithmetic_pins_operand_layouts():
+    # integer scores with scale*log2e = 1: P is a power of two (exact in fp16), V integer: only the fp16 output
+    # rounds, so a wrong key <-> V-row association or a transposed operand cannot hide inside the tolerance
+    rng = np.random.default_rng(11)
+    for D in (64, 128, 256):
+        B, S, H = 1, 384, 2
+        q = np.zeros((B, S, H, D), np.float32)
+        np.put_along_axis(q, rng.integers(0, D, (B, S, H, 4)), 1.0, axis=-1)
+        k = rng.integers(-1, 2, (B, S, H, D)).astype(np.float32)
+        v = rng.integers(-8, 9, (B, S, H, D)).astype(np.float32)
+        got, (qf, kf, vf) = _run(q, k, v, softmax_scale=float(np.log(2.0)))
+        ref = oracle.attention_f32(qf, kf, vf, alpha0=np.log(2.0))["O"]
+        np.testing.assert_allclose(got, ref, rtol=1.5e-3, atol=2e-4)
+
+
 def test_nondefault_scale():
     _check_full(1, 256, 2, 128, scale=0.05)
 

@@ -1,0 +1,145 @@
+"""GPU parity of the fp8 e4m3 FMHA forward (through the C-ABI) against the CPU oracle run on the DEQUANTISED
+operands, as the reference's own check does (src/fmha-pipeline/fmha_forward.cu:613-631).  Gates: max-abs error
+<= 5e-2, and the reference's error-percentage criterion at its fp8 threshold (fmha_forward.cu:638-639)."""
+import numpy as np
+import pytest
+
+import oracle
+from _util import ERRPCT_FP8, TOL_FP8, max_abs, pkg, subset_pairs, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _quant(x, per_tensor=True):
+    if per_tensor:
+        codes, scale = oracle.quantize_e4m3_per_tensor(x)
+    else:  # the reference's mode: values cast straight to e4m3, no scales (fmha_forward.cu:498-500)
+        codes, scale = oracle.e4m3_encode(x), np.float32(1.0)
+    return codes, float(scale), oracle.e4m3_decode(codes) * scale
+
+
+def _run(q, k, v, per_tensor=True, **kw):
+    import torch
+    (qc, qs, qf), (kc, ks, kf), (vc, vs, vf) = (_quant(x, per_tensor) for x in (q, k, v))
+    o = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(vc), q_descale=qs, k_descale=ks, v_descale=vs, **kw)
+    torch.cuda.synchronize()
+    return o.float().cpu().numpy(), (qf, kf, vf)
+
+
+def _check_full(B, S, H, D, per_tensor=True, seqlen_kv=None):
+    q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=seqlen_kv)
+    got, (qf, kf, vf) = _run(q, k, v, per_tensor)
+    ref = oracle.attention_f32(qf, kf, vf)["O"]
+    err = max_abs(got, ref)
+    ok, pct = oracle.verify_tensor(got, ref, ERRPCT_FP8)
+    print(f"fp8 B={B} S={S}/{seqlen_kv or S} H={H} D={D} per_tensor={per_tensor}: max-abs {err:.3e}, error% {pct:.2e}")
+    assert err <= TOL_FP8, err
+    # The reference's percentage criterion is calibrated for its own problem size (S = 4096, where the e4m3
+    # rounding noise of P averages over thousands of keys): it is enforced from S >= 2048 on; the short shapes
+    # here are held to the max-abs gate and to the e4m3-P emulation test below.
+    if S >= 2048 and (seqlen_kv or S) >= 2048:
+        assert ok, pct
+    return got, ref
+
+
+@pytest.mark.parametrize("B,S,H", [(1, 256, 2), (2, 512, 3), (1, 1024, 4), (1, 4096, 2)])
+def test_small_shapes_per_tensor_scales(B, S, H):
+    _check_full(B, S, H, 128)
+
+
+def test_reference_mode_unit_scales():
+    _check_full(1, 512, 2, 128, per_tensor=False)
+
+
+def test_rectangular_q_kv():
+    _check_full(1, 256, 2, 128, seqlen_kv=640)
+    _check_full(1, 512, 2, 128, seqlen_kv=128)
+
+
+def test_matches_tiled_emulation_with_e4m3_p():
+    # against the numpy emulation of the kernel-side algorithm with P rounded to e4m3 the kernel agrees far more
+    # closely than against the fp32 attention: what is left is P's bias (a power of two) and fp16 output rounding
+    B, S, H, D = 1, 256, 1, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    got, (qf, kf, vf) = _run(q, k, v)
+    ref = oracle.attention_f32(qf, kf, vf)["O"]
+    emu, _, _ = oracle.online_softmax_tiled(qf[0, :, 0], kf[0, :, 0], vf[0, :, 0], 64, oracle.LOG2E / np.sqrt(D),
+                                            p_cast="e4m3")
+    e_ref, e_emu = max_abs(got[0, :, 0], ref[0, :, 0]), max_abs(got[0, :, 0], emu)
+    print(f"vs fp32 attention {e_ref:.3e}; vs e4m3-P emulation {e_emu:.3e}")
+    assert e_ref <= TOL_FP8 and e_emu <= TOL_FP8
+
+
+def test_exact_arithmetic_pins_the_v_layout_transform():
+    # Exact-arithmetic mode (the reference's integer-input trick, include/utils/random.hpp:13-32, taken one step
+    # further): integer scores with scale*log2e = 1 make every P a power of two, exactly representable in e4m3,
+    # and integer V in [-8, 8] is exact too -- so the fp8 kernel has NO rounding left but the fp16 output, and any
+    # wrong key <-> V-row association in the tr8 operand transform shows up at full size.
+    rng = np.random.default_rng(11)
+    B, S, H, D = 1, 512, 2, 128
+    q = np.zeros((B, S, H, D), np.float32)
+    idx = rng.integers(0, D, (B, S, H, 4))
+    np.put_along_axis(q, idx, 1.0, axis=-1)                       # up to four ones per query row
+    k = rng.integers(-1, 2, (B, S, H, D)).astype(np.float32)      # scores are integers in [-4, 4]
+    v = rng.integers(-8, 9, (B, S, H, D)).astype(np.float32)
+    got, (qf, kf, vf) = _run(q, k, v, per_tensor=False, softmax_scale=float(np.log(2.0)))
+    assert np.array_equal(qf, q) and np.array_equal(kf, k) and np.array_equal(vf, v)
+    ref = oracle.attention_f32(qf, kf, vf, alpha0=np.log(2.0))["O"]
+    np.testing.assert_allclose(got, ref, rtol=1.5e-3, atol=2e-4)
+
+
+def test_taps_and_invariants():
+    import torch
+    B, S, H, D = 1, 512, 2, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    rm = torch.full((B, H, S), -1.0, dtype=torch.float32, device="cuda:0")
+    rs = torch.full((B, H, S), -1.0, dtype=torch.float32, device="cuda:0")
+    base, (qf, kf, vf) = _run(q, k, v, row_max=rm, row_sum=rs)
+    r = oracle.attention_f32(qf, kf, vf, want_stats=True)
+    # max-check / sum-check (fmha_forward.cu:655-676); scores are exact products of e4m3 values in fp32
+    np.testing.assert_allclose(rm.cpu().numpy() / oracle.LOG2E, r["row_max"], rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(1.0 / rs.cpu().numpy(), r["inv_sum"], rtol=1e-3)
+    # V = 1 -> O ~ 1 (P is rounded to e4m3 after the fp32 row sum)
+    ones, _ = _run(q, k, np.ones_like(v))
+    assert max_abs(ones, 1.0) <= 2e-2
+    # a common permutation of the keys (pins the V-tile layout transform: wrong key order in V would show here
+    # and in every other test)
+    perm = np.random.default_rng(5).permutation(S)
+    permd, _ = _run(q, k[:, perm], v[:, perm])
+    assert max_abs(base, permd) <= 2e-2
+    # one dominant key selects its V row exactly (e4m3 V values are exact in fp16)
+    qd = np.zeros_like(q)
+    qd[..., 0] = 300.0
+    kd = np.zeros_like(k)
+    kd[0, 77, :, 0] = 300.0
+    sel, (_, _, vf2) = _run(qd, kd, v)
+    np.testing.assert_allclose(sel[0, :, 0], np.broadcast_to(vf2[0, 77, 0], sel[0, :, 0].shape), rtol=2e-3, atol=1e-4)  # fp16 output rounding only
+
+
+def test_unsupported_modes_report_errors():
+    import torch
+    x = torch.zeros((1, 128, 1, 64), dtype=torch.uint8, device="cuda:0")
+    with pytest.raises(pkg.CfkError) as e:
+        pkg.fmha_forward(x, x, x)
+    assert e.value.code == -2
+
+
+def test_config4_subset_check():
+    # BASELINE config 4: fp8 e4m3 B=4 H=16 S=4096 D=128, per-tensor amax scales, V in [B,S,H,D]
+    B, S, H, D = 4, 4096, 16, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    got, (qf, kf, vf) = _run(q, k, v)
+    pairs = subset_pairs(B, H)
+    ref = oracle.attention_f32(qf, kf, vf, bh_pairs=pairs)["O"]
+    oracle.attention_f32(qf, kf, vf, bh_pairs=[(b, h) for b in range(B) for h in range(H)], row_start=17,
+                         row_step=61, out=ref)
+    sel = ~np.isnan(ref)
+    err = max_abs(got[sel], ref[sel])
+    ok, pct = oracle.verify_tensor(got[sel], ref[sel], ERRPCT_FP8)
+    # for information: error against the attention of the UNQUANTISED tensors
+    full = oracle.attention_f32(q, k, v, bh_pairs=pairs[:1])["O"]
+    s1 = ~np.isnan(full)
+    print(f"fp8 cfg4: checked {sel.sum()} elements, max-abs {err:.3e}, error% {pct:.2e}; "
+          f"vs unquantised fp32 attention {max_abs(got[s1], full[s1]):.3e}")
+    assert err <= TOL_FP8 and ok
+    assert not np.any(np.isnan(got))
