@@ -1,0 +1,77 @@
+"""The C++ bench/test driver (cutlass-kernels_amd/driver/fmha_forward): command line of the reference driver
+(src/fmha-pipeline/fmha_forward.cu:687-794), its check lines, and an independent check of what it dumps."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import oracle
+from _util import ERRPCT_FP16, ERRPCT_FP8, ROOT, TOL_FP16, TOL_FP8, max_abs
+
+DRIVER = os.path.join(ROOT, "cutlass-kernels_amd", "driver", "fmha_forward")
+
+
+def _run(*args, check=True):
+    r = subprocess.run([DRIVER, *args], capture_output=True, text=True, timeout=600)
+    if check:
+        assert r.returncode == 0, r.stdout + r.stderr
+    return r
+
+
+def test_driver_is_built():
+    assert os.path.exists(DRIVER), "build it: python -c 'import __graft_entry__ as g; g.build()'"
+
+
+def test_usage_and_flag_errors_without_gpu():
+    out = _run("--help").stdout
+    for flag in ("--prec-type", "--batch-size", "--dim-size", "--head-size", "--seq-length", "--iterations",
+                 "--num-cuda-streams", "--reference-check", "--print-values"):
+        assert flag in out
+    r = _run("--head-size=96", check=False)
+    assert r.returncode != 0 and "Unsupported head dim: 96" in r.stdout
+    r = _run("--prec-type=3", check=False)
+    assert r.returncode != 0 and "Unsupported type: 3" in r.stdout
+    r = _run("--batch-size=2", "--num-cuda-streams=4", check=False)
+    assert r.returncode != 0 and "max no. of cuda streams" in r.stdout
+
+
+def test_driver_e4m3_encoder_matches_codec():
+    lines = _run("--selftest-e4m3").stdout.split()
+    bits = np.array([int(x, 16) for x in lines[0::2]], dtype=np.uint32)
+    codes = np.array([int(x, 16) for x in lines[1::2]], dtype=np.uint8)
+    assert bits.size == 4096
+    assert np.array_equal(codes, oracle.e4m3_encode(bits.view(np.float32)))
+
+
+def _load_dump(d):
+    meta = dict(l.split() for l in open(os.path.join(d, "meta.txt")).read().strip().splitlines())
+    B, S, H, D, prec = (int(meta[k]) for k in ("B", "S", "H", "D", "prec"))
+    shape = (B, S, H, D)
+    if prec == 1:
+        q, k, v = (np.fromfile(os.path.join(d, f + ".bin"), dtype=np.float16).reshape(shape).astype(np.float32)
+                   for f in "qkv")
+    else:
+        q, k, v = (oracle.e4m3_decode(np.fromfile(os.path.join(d, f + ".bin"), dtype=np.uint8).reshape(shape)) *
+                   np.float32(meta[f + "_descale"]) for f in "qkv")
+    o = np.fromfile(os.path.join(d, "o.bin"), dtype=np.float16).reshape(shape).astype(np.float32)
+    return q, k, v, o, prec
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("prec,head,extra", [(1, 64, []), (1, 128, ["--num-cuda-streams=2"]), (1, 256, []),
+                                             (2, 128, []), (2, 128, ["--fp8-scales=amax"])])
+def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
+    # fp8 needs the reference's own sequence length for its percentage criterion; fp16 passes at any length
+    seq = 2048 if prec == 2 else 512
+    out = _run(f"--prec-type={prec}", "--batch-size=2", f"--dim-size={2 * head}", f"--head-size={head}",
+               f"--seq-length={seq}", "--iterations=3", "--reference-check=true", "--verify-all=true",
+               f"--dump-dir={tmp_path}", *extra).stdout
+    assert "CUTE_FMHA:" in out and "Gflop/s" in out
+    assert "gemm-check-2: Passed" in out and "max-check: Passed" in out and "sum-check: Passed" in out
+    assert f"K = {head}" in out and "QBLK = " in out
+    # independent check of the dumped tensors against the CPU oracle
+    q, k, v, o, p = _load_dump(str(tmp_path))
+    ref = oracle.attention_f32(q, k, v)["O"]
+    assert max_abs(o, ref) <= (TOL_FP16 if p == 1 else TOL_FP8)
+    assert oracle.verify_tensor(o, ref, ERRPCT_FP16 if p == 1 else ERRPCT_FP8)[0]
