@@ -23,6 +23,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"f16": 2500.0, "f8": 5000.0}   # MI355X published dense MFMA peaks
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the same
+# counter reads for a plain 256 MiB copy: FETCH x2.0, WRITE x1.0); summaries are under profiles/.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {"cfg2": (196792 + 65550) * 1024, "cfg4": (98464 + 65544) * 1024}
 
 WORKLOADS = {
     "cfg1": dict(kind="fmha", dtype="f16", B=1, H=8, S=512, D=64, scale=0.125),
@@ -188,7 +191,8 @@ def main():
         "config": {"workload": main_res["workload"], "flop_per_step": main_res["flop_per_step"],
                    "layout": "[B,S,H,D]", "seeds": [3081, 3082, 3083]},
         "roofline": {"bound": "mfma", "achieved": main_res["tflops"], "peak": main_res["peak_tflops"],
-                     "unit": "TFLOP/s", "frac": main_res["frac_of_peak"], "traffic": None},
+                     "unit": "TFLOP/s", "frac": main_res["frac_of_peak"],
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
         "secondary": secondary,
     }
     if not args.no_cpu_baseline and w["kind"] == "fmha":
