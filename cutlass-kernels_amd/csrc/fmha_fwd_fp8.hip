@@ -56,16 +56,28 @@ struct Fp8Cfg {
   static constexpr int CPR = D / 16;                     // 16-byte chunks per row
   static constexpr int RPI = 1024 / PITCH;               // rows per wave-wide 16 B/lane copy
   static constexpr int IPW = BN / RPI / NWAVES;          // copies per wave per tile
-  static_assert(D == 128, "fp8 kernel is built for head dim 128");
+  static_assert(D == 64 || D == 128 || D == 256, "head dim");
   static_assert(BN % (RPI * NWAVES) == 0 && IPW >= 1, "tile must split evenly over the waves");
 };
 
-// XOR swizzles of the 16-byte chunk index (rows are 128 B, LDS banks repeat every 256 B, so two rows share a
-// bank period).  K: ds_read_b128 by 16 consecutive rows at one chunk index -> the 8 rows of equal parity need 8
-// distinct values.  V: ds_read_b64_tr_b8 by keys {4g..4g+3, 8+4g..8+4g+3} x 32 contiguous bytes -> the 4 keys of
-// equal parity need 4 distinct 32-byte slots; bit 0 stays clear so a 32-byte pair stays contiguous.
-__device__ __forceinline__ int swz_k8(int row) { return (row >> 1) & 7; }
-__device__ __forceinline__ int swz_v8(int row) { return (((row >> 1) & 1) << 1) | (((row >> 3) & 1) << 2); }
+// XOR swizzles of the 16-byte chunk index of a row (rows are D bytes; LDS banks repeat every 256 B, so 256/D rows
+// share a bank period).
+//  K: ds_read_b128 by 16 consecutive rows at one chunk index -> the rows that share a position inside the bank
+//     period (16*D/256 of them) need distinct XOR values.
+//  V: ds_read_b64_tr_b8 by keys {4g..4g+3, 8+4g..8+4g+3} x 32 contiguous bytes -> keys that share a position
+//     inside the bank period need distinct 32-byte slots; bit 0 stays clear so a 32-byte pair stays contiguous.
+template <int D>
+__device__ __forceinline__ int swz_k8(int row) {
+  if (D == 64) return (row >> 2) & 3;
+  if (D == 128) return (row >> 1) & 7;
+  return ((row & 3) << 2) | ((row >> 2) & 3);
+}
+template <int D>
+__device__ __forceinline__ int swz_v8(int row) {
+  if (D == 64) return ((row >> 3) & 1) << 1;
+  if (D == 128) return (((row >> 1) & 1) << 1) | (((row >> 3) & 1) << 2);
+  return ((row & 3) | (((row >> 3) & 1) << 2)) << 1;
+}
 
 template <class C>
 __global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(C::WPE, C::WPE)))
@@ -106,8 +118,8 @@ fmha_fwd_fp8_kernel(const FmhaArgs a) {
   for (int i = 0; i < C::IPW; ++i) {
     const int row = (i * C::NWAVES + wave) * C::RPI + lane / C::CPR;
     const int cp = lane % C::CPR;
-    goff_k[i] = (uint32_t)row * ld_bytes + (uint32_t)((cp ^ swz_k8(row)) * 16);
-    goff_v[i] = (uint32_t)row * ld_bytes + (uint32_t)((cp ^ swz_v8(row)) * 16);
+    goff_k[i] = (uint32_t)row * ld_bytes + (uint32_t)((cp ^ swz_k8<D>(row)) * 16);
+    goff_v[i] = (uint32_t)row * ld_bytes + (uint32_t)((cp ^ swz_v8<D>(row)) * 16);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
   auto load_tile = [&](const char *gbase, const uint32_t (&goff)[C::IPW], int jt, int lds_off) {
@@ -132,7 +144,7 @@ fmha_fwd_fp8_kernel(const FmhaArgs a) {
 #pragma unroll
   for (int s = 0; s < KS; ++s)
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh) k_rd[s][hh] = r * C::PITCH + (((4 * s + 2 * g + hh) ^ swz_k8(r)) * 16);
+    for (int hh = 0; hh < 2; ++hh) k_rd[s][hh] = r * C::PITCH + (((4 * s + 2 * g + hh) ^ swz_k8<D>(r)) * 16);
   // V operand via ds_read_b64_tr_b8 (see the file comment)
   const int li = lane & 15;
   const int row_e = li >> 1;
@@ -141,7 +153,7 @@ fmha_fwd_fp8_kernel(const FmhaArgs a) {
 #pragma unroll
   for (int db = 0; db < DB; ++db) {
     const int c = 2 * db + ((lane >> 4) & 1);
-    v_rd[db] = v_key * C::PITCH + ((c ^ swz_v8(v_key)) * 16) + 8 * (li & 1);
+    v_rd[db] = v_key * C::PITCH + ((c ^ swz_v8<D>(v_key)) * 16) + 8 * (li & 1);
   }
 
   f32x16 oacc[DB];
@@ -293,16 +305,18 @@ hipError_t launch_cfg(const FmhaArgs &a, hipStream_t s) {
   return hipGetLastError();
 }
 
+using Cfg64S = Fp8Cfg<64, 4, 2>;
 using Cfg128S = Fp8Cfg<128, 4, 2>;
 using Cfg128L = Fp8Cfg<128, 8, 2>;
+using Cfg256S = Fp8Cfg<256, 4, 1>;   // O (128) + S (64) + Q (32) registers: one wave per SIMD
 
-bool use_large(int sq, int bh) {
+bool use_large(int head_dim, int sq, int bh) {
   static const int forced = [] {
     const char *e = getenv("CFK_FMHA_TILE");
     if (!e) return -1;
     return e[0] == 's' ? 0 : e[0] == 'l' ? 1 : -1;
   }();
-  if (sq % 256 != 0 || forced == 0) return false;
+  if (head_dim != 128 || sq % 256 != 0 || forced == 0) return false;
   if (forced == 1) return true;
   return (long long)bh * (sq / 256) >= 512;
 }
@@ -316,19 +330,29 @@ void fill_plan(int sq, int bh, FmhaPlan *p) {
   p->grid = bh * (sq / C::BM);
 }
 
+template <class F>
+bool dispatch(int head_dim, int sq, int bh, F &&f) {
+  switch (head_dim) {
+    case 64: f(Cfg64S{}); return true;
+    case 128: use_large(head_dim, sq, bh) ? f(Cfg128L{}) : f(Cfg128S{}); return true;
+    case 256: f(Cfg256S{}); return true;
+    default: return false;
+  }
+}
+
 }  // namespace
 
 bool plan_fmha_fp8(int head_dim, int sq, int skv, int bh, int v_layout, FmhaPlan *p) {
   (void)skv;
-  if (head_dim != 128 || v_layout != 0) return false;
-  if (use_large(sq, bh)) fill_plan<Cfg128L>(sq, bh, p);
-  else fill_plan<Cfg128S>(sq, bh, p);
-  return true;
+  if (v_layout != 0) return false;
+  return dispatch(head_dim, sq, bh, [&](auto cfg) { fill_plan<decltype(cfg)>(sq, bh, p); });
 }
 
 hipError_t launch_fmha_fp8(const FmhaArgs &a, int head_dim, hipStream_t s) {
-  if (head_dim != 128 || a.v_layout != 0) return hipErrorNotSupported;
-  return use_large(a.Sq, a.B * a.H) ? launch_cfg<Cfg128L>(a, s) : launch_cfg<Cfg128S>(a, s);
+  if (a.v_layout != 0) return hipErrorNotSupported;
+  hipError_t e = hipErrorNotSupported;
+  dispatch(head_dim, a.Sq, a.B * a.H, [&](auto cfg) { e = launch_cfg<decltype(cfg)>(a, s); });
+  return e;
 }
 
 }  // namespace cfk

@@ -15,8 +15,7 @@ STATUS=0
 for TILE in "${TILES[@]}"; do
 for PREC in "${PRECS[@]}"; do
 for HEAD in "${HEADSIZES[@]}"; do
-  if [[ $PREC == 2 && $HEAD != 128 ]]; then continue; fi   # fp8 is built for head size 128
-  if [[ $TILE == large && $HEAD == 256 ]]; then continue; fi
+  if [[ $TILE == large && ( $HEAD == 256 || ( $PREC == 2 && $HEAD == 64 ) ) ]]; then continue; fi   # no large tile there
   export CFK_FMHA_TILE=$TILE
   if [[ $MODE == verify || $MODE == verify-all ]]; then
     VA=false; [[ $MODE == verify-all ]] && VA=true

@@ -60,7 +60,7 @@ def _load_dump(d):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("prec,head,extra", [(1, 64, []), (1, 128, ["--num-cuda-streams=2"]), (1, 256, []),
-                                             (2, 128, []), (2, 128, ["--fp8-scales=amax"])])
+                                             (2, 128, []), (2, 128, ["--fp8-scales=amax"]), (2, 64, []), (2, 256, [])])
 def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
     # fp8 needs the reference's own sequence length for its percentage criterion; fp16 passes at any length
     seq = 2048 if prec == 2 else 512

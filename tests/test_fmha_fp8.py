@@ -42,9 +42,10 @@ def _check_full(B, S, H, D, per_tensor=True, seqlen_kv=None):
     return got, ref
 
 
-@pytest.mark.parametrize("B,S,H", [(1, 256, 2), (2, 512, 3), (1, 1024, 4), (1, 4096, 2)])
-def test_small_shapes_per_tensor_scales(B, S, H):
-    _check_full(B, S, H, 128)
+@pytest.mark.parametrize("B,S,H,D", [(1, 256, 2, 128), (2, 512, 3, 128), (1, 1024, 4, 128), (1, 4096, 2, 128),
+                                     (2, 512, 3, 64), (1, 4096, 2, 64), (2, 384, 2, 256), (1, 4096, 1, 256)])
+def test_shapes_per_tensor_scales(B, S, H, D):
+    _check_full(B, S, H, D)
 
 
 def test_reference_mode_unit_scales():
@@ -76,16 +77,17 @@ def test_exact_arithmetic_pins_the_v_layout_transform():
     # and integer V in [-8, 8] is exact too -- so the fp8 kernel has NO rounding left but the fp16 output, and any
     # wrong key <-> V-row association in the tr8 operand transform shows up at full size.
     rng = np.random.default_rng(11)
-    B, S, H, D = 1, 512, 2, 128
-    q = np.zeros((B, S, H, D), np.float32)
-    idx = rng.integers(0, D, (B, S, H, 4))
-    np.put_along_axis(q, idx, 1.0, axis=-1)                       # up to four ones per query row
-    k = rng.integers(-1, 2, (B, S, H, D)).astype(np.float32)      # scores are integers in [-4, 4]
-    v = rng.integers(-8, 9, (B, S, H, D)).astype(np.float32)
-    got, (qf, kf, vf) = _run(q, k, v, per_tensor=False, softmax_scale=float(np.log(2.0)))
-    assert np.array_equal(qf, q) and np.array_equal(kf, k) and np.array_equal(vf, v)
-    ref = oracle.attention_f32(qf, kf, vf, alpha0=np.log(2.0))["O"]
-    np.testing.assert_allclose(got, ref, rtol=1.5e-3, atol=2e-4)
+    for D in (64, 128, 256):
+        B, S, H = 1, 512, 2
+        q = np.zeros((B, S, H, D), np.float32)
+        idx = rng.integers(0, D, (B, S, H, 4))
+        np.put_along_axis(q, idx, 1.0, axis=-1)                       # up to four ones per query row
+        k = rng.integers(-1, 2, (B, S, H, D)).astype(np.float32)      # scores are integers in [-4, 4]
+        v = rng.integers(-8, 9, (B, S, H, D)).astype(np.float32)
+        got, (qf, kf, vf) = _run(q, k, v, per_tensor=False, softmax_scale=float(np.log(2.0)))
+        assert np.array_equal(qf, q) and np.array_equal(kf, k) and np.array_equal(vf, v)
+        ref = oracle.attention_f32(qf, kf, vf, alpha0=np.log(2.0))["O"]
+        np.testing.assert_allclose(got, ref, rtol=1.5e-3, atol=2e-4)
 
 
 def test_taps_and_invariants():
@@ -119,8 +121,9 @@ def test_taps_and_invariants():
 def test_unsupported_modes_report_errors():
     import torch
     x = torch.zeros((1, 128, 1, 64), dtype=torch.uint8, device="cuda:0")
+    xt = torch.zeros((1, 64, 1, 128), dtype=torch.uint8, device="cuda:0")
     with pytest.raises(pkg.CfkError) as e:
-        pkg.fmha_forward(x, x, x)
+        pkg.fmha_forward(x, x, xt, v_layout=pkg.fmha.CFK_V_BDHS)   # pre-transposed V is not built
     assert e.value.code == -2
 
 
