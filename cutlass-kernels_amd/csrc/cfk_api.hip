@@ -39,21 +39,22 @@ int check_fmha(const cfk_fmha_fwd_params *p, cfk::FmhaPlan *plan, bool need_poin
     return fail(CFK_ERR_UNSUPPORTED, "Unsupported head dim: %d", p->head_dim);
   if (p->v_layout != CFK_V_BSHD && p->v_layout != CFK_V_BDHS)
     return fail(CFK_ERR_INVALID_ARG, "unknown v_layout %d", p->v_layout);
-  if (p->dtype != p->v_dtype)
-    return fail(CFK_ERR_UNSUPPORTED, "hybrid precision (Q,K fp8 with fp16 P,V) is not built; v_dtype must equal dtype");
-  if (p->dtype == CFK_FP16 && p->v_layout != CFK_V_BSHD)
-    return fail(CFK_ERR_UNSUPPORTED, "pre-transposed V ([B,D,H,S]) is accepted for fp8 only");
+  if (p->dtype == CFK_FP16 && p->v_dtype != CFK_FP16)
+    return fail(CFK_ERR_UNSUPPORTED, "fp16 Q,K with fp8 V is not a mode of the reference; v_dtype must be fp16");
+  if (p->v_dtype == CFK_FP16 && p->v_layout != CFK_V_BSHD)
+    return fail(CFK_ERR_UNSUPPORTED, "pre-transposed V ([B,D,H,S]) is an fp8-V layout");
   if (!(p->softmax_scale > 0.f) || !std::isfinite(p->softmax_scale))
     return fail(CFK_ERR_INVALID_ARG, "softmax_scale must be positive and finite");
   if (p->dtype == CFK_FP8_E4M3) {
-    const float d[3] = {p->q_descale, p->k_descale, p->v_descale};
+    const float d[3] = {p->q_descale, p->k_descale, p->v_dtype == CFK_FP8_E4M3 ? p->v_descale : 1.0f};
     for (float x : d)
       if (!(x > 0.f) || !std::isfinite(x)) return fail(CFK_ERR_INVALID_ARG, "fp8 descales must be positive and finite");
   }
   const long long bh = (long long)p->batch * p->heads;
   if (bh > (1 << 24)) return fail(CFK_ERR_UNSUPPORTED, "batch*heads too large");
-  bool ok = p->dtype == CFK_FP16 ? cfk::plan_fmha_f16(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, plan)
-                                 : cfk::plan_fmha_fp8(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, p->v_layout, plan);
+  bool ok = p->dtype == CFK_FP16     ? cfk::plan_fmha_f16(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, plan)
+            : p->v_dtype == CFK_FP16 ? cfk::plan_fmha_hybrid(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, plan)
+                                     : cfk::plan_fmha_fp8(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, p->v_layout, plan);
   if (!ok) return fail(CFK_ERR_UNSUPPORTED, "no kernel for dtype %d head dim %d v_layout %d", p->dtype, p->head_dim, p->v_layout);
   // The kernels carry no masks, exactly like the reference (no bounds handling: fmha_forward.cu:361-372).
   if (p->seqlen_q % plan->block_m != 0)
@@ -125,6 +126,10 @@ int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
     a.scale_log2 = p->softmax_scale * kLog2e;
     a.out_scale = 1.0f;
     e = cfk::launch_fmha_f16(a, p->head_dim, (hipStream_t)stream);
+  } else if (p->v_dtype == CFK_FP16) {  // hybrid: fp16 V carries no scale
+    a.scale_log2 = p->softmax_scale * kLog2e * p->q_descale * p->k_descale;
+    a.out_scale = 1.0f;
+    e = cfk::launch_fmha_hybrid(a, p->head_dim, (hipStream_t)stream);
   } else {
     a.scale_log2 = p->softmax_scale * kLog2e * p->q_descale * p->k_descale;
     a.out_scale = p->v_descale;

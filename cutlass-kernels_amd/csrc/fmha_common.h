@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <cstdlib>
+
 namespace cfk {
 
 // Argument block handed to every FMHA kernel (by value).  Tensors are [B, S, H, D] with D contiguous, the
@@ -23,10 +25,12 @@ struct FmhaPlan {
 };
 
 // Each launcher validates nothing: the C-ABI layer has already checked shapes against the plan.
-hipError_t launch_fmha_f16(const FmhaArgs &a, int head_dim, hipStream_t s);
-hipError_t launch_fmha_fp8(const FmhaArgs &a, int head_dim, hipStream_t s);
+hipError_t launch_fmha_f16(const FmhaArgs &a, int head_dim, hipStream_t s);      // Q,K,V fp16
+hipError_t launch_fmha_fp8(const FmhaArgs &a, int head_dim, hipStream_t s);      // Q,K,V e4m3, P e4m3
+hipError_t launch_fmha_hybrid(const FmhaArgs &a, int head_dim, hipStream_t s);   // Q,K e4m3; P,V fp16
 bool plan_fmha_f16(int head_dim, int sq, int skv, int bh, FmhaPlan *p);
 bool plan_fmha_fp8(int head_dim, int sq, int skv, int bh, int v_layout, FmhaPlan *p);
+bool plan_fmha_hybrid(int head_dim, int sq, int skv, int bh, FmhaPlan *p);
 
 hipError_t launch_gemm_f16(int M, int N, int K, const void *A, const void *B, void *C, int layout, hipStream_t s);
 
@@ -40,5 +44,16 @@ __device__ __forceinline__ int xcd_remap(int wg, int n) {
   if (wg >= main_n) return wg;  // ragged tail keeps its id
   return (wg % kXcds) * per + wg / kXcds;
 }
+
+#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T *)(p))
+
+// Asynchronous 16 B/lane global -> LDS copy: lane l writes LDS bytes [lds_addr + 16 l, +16) with the 16 bytes at
+// its own global address.  Issued through inline asm on purpose: the compiler then does not track the copy, so it
+// does not drain vmcnt before every later LDS read, and the copies of one pipeline step stay in flight until
+// the explicit wait_lds_dma() in front of the step's closing barrier.  lds_addr must be wave-uniform.
+__device__ __forceinline__ void lds_dma16(const void *gptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void wait_lds_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 }  // namespace cfk

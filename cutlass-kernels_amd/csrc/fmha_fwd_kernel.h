@@ -1,0 +1,420 @@
+// The FMHA forward kernel for gfx950 (MI355X), one template for the three precision modes of the reference:
+//   fp16            Q,K,V fp16                      (--prec-type=1)
+//   fp8             Q,K,V e4m3, P cast to e4m3      (--prec-type=2 built with -DGEMM2FP8, fmha_forward.cu:446-450)
+//   hybrid          Q,K e4m3; P,V fp16              (--prec-type=2 without GEMM2FP8, the reference's default fp8 build)
+// always fp32 softmax / accumulation and fp16 output.
+//
+// Takes the place of the reference's device kernels fmhaForwardPipelinedNoWspl / ...Wspl / fmhaForwardNoPipeline
+// (src/fmha-pipeline/fmha_pipe_nows.h:72-331, fmha_pipe_ws.h:69-365, fmha_nopipe.h:43-342) and of their building
+// blocks fmhaForwardProducer (fmha_producer.h:4-79), fmhaForwardConsumer (fmha_consumer.h:8-73),
+// onlineSoftmaxAndRescale (online_softmax.h:87-207), applySoftmaxNormalizer (online_softmax.h:59-85), convert_type /
+// ReorgCFp8toAFp8 (reg2reg.h:18-108), the epilogue (fmha_epilogue.h:120-177), the tile constants
+// (shared_storage.h:4-85) and the MMA selectors (ss_helper.h:3-94).  Same mathematics, different machine mapping:
+//
+//  * One workgroup owns BM = NWAVES*32 query rows of one (batch, head); a wave owns 32 rows; key tiles of BN keys.
+//  * Both GEMMs run TRANSPOSED on 32x32 MFMAs (v_mfma_f32_32x32x16_f16, or v_mfma_f32_32x32x64_f8f6f4 for e4m3 -- the
+//    legacy fp8 MFMA only runs at the fp16 rate):
+//        S^T[key, q] = K[key, :] . Q[q, :]       A = K tile from LDS (ds_read_b128), B = Q resident in VGPRs
+//        O^T[d,  q] += V^T[d, key] . P^T[key, q]  A = V tile read TRANSPOSED from LDS, B = P straight from the S^T
+//                                                 accumulator registers.
+//    In the 32x32 accumulator layout lane (q = lane%32, g = lane/32) holds rows 8*(v/4)+4*g+(v%4), v = 0..15, of
+//    column q: one lane holds 16 keys of ONE query.  Row max / row sum are in-lane reductions plus one exchange with
+//    lane^32; running max / sum / rescale factor are per-lane scalars; and the accumulator registers, cast to the P
+//    precision, already ARE the B operand of the second MFMA under a fixed permutation of the keys of a K-step.  The
+//    permutation is applied to V instead (a GEMM is invariant under a common permutation of its contraction index):
+//    it falls out of the per-lane addresses handed to the LDS transpose reads.  P never crosses lanes, never touches
+//    LDS (the reference shuffles across the quad, online_softmax.h:39-57 and reg2reg.h:71-107).
+//      - fp16 V: ds_read_b64_tr_b16 hands a lane 4 consecutive keys of one head-dim column.
+//      - e4m3 V, "the fp8 V-tile layout transform": the A operand needs per lane (d, g) the 32 bytes V[key(t,g)][d],
+//        slot t = key 32*(t/16) + 8*((t%16)/4) + 4*g + t%4 -- a byte transpose plus that key permutation.  Four
+//        ds_read_b64_tr_b8 deliver it: in a block of 16 lanes, lane L supplies the address of (row L/2, 8-byte column
+//        group L%2) and lane i receives rows 0..7 of column i; row e of load u is pointed at key 16u+8(e/4)+4g+e%4.
+//        V stays [B,S,H,D] in HBM: no host transpose (fmha_forward.cu:514-532), no host permutation (:534-558).
+//  * K/V tiles go global -> LDS directly (global_load_lds_dwordx4, no VGPR staging), two stages each.  Rows are
+//    unpadded; bank conflicts are removed by XOR-swizzling the 16-byte chunks of a row on the GLOBAL side of the
+//    copy (lane i of a copy always writes LDS slot i, but may fetch any chunk).
+//  * Software pipeline (the reference overlaps only TMA with compute; its GEMMs drain the MMA pipe,
+//    lib/gemm/gemm_tensor.hpp:14-25): step j issues S_{j+1} = K_{j+1}.Q^T on the MFMA pipe while the VALU does
+//    exp2 / row sum / cast of S_j, then O += P_j.V_j while the VALU finds the row max of S_{j+1}.  S lives in two
+//    register sets that swap roles every step (the loop is unrolled by two).
+//  * Deferred rescale: the reference rescales O and l by exp2(m_old - m_new) on every tile (online_softmax.h:
+//    144-165).  Any reference point m_ref works as long as exp2(t - m_ref) stays representable, so m_ref only moves
+//    -- and O, l are only rescaled -- when a tile max exceeds it by more than kTau = 8 (P <= 256 fits fp16 and
+//    e4m3).  With e4m3 P the reference point additionally sits 7 below the row max, so P spans (0, 2^8] instead of
+//    (0, 1] and probabilities down to 2^-17 of the row max stay out of e4m3's flush zone (the reference casts P in
+//    (0,1] directly, fmha_consumer.h:54); the bias cancels in O/l.
+//  * Per-tensor fp8 scales: q_descale*k_descale is folded into the exp2 scale, v_descale into the final 1/l.
+//  * Workgroup ids are remapped so the query blocks of one head share an XCD's L2.
+#pragma once
+#include <type_traits>
+
+#include "fmha_common.h"
+
+namespace cfk {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef int int8v __attribute__((ext_vector_type(8)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int2v __attribute__((ext_vector_type(2)));
+
+template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_>
+struct FmhaCfg {
+  static constexpr int D = D_, BN = BN_, NWAVES = NWAVES_;
+  static constexpr int WPE = WPE_;                              // waves per SIMD the register budget is sized for
+  static constexpr bool QK8 = QK8_, PV8 = PV8_;                 // e4m3 (true) or fp16 (false) operands of GEMM-I / II
+  static constexpr int T = NWAVES * 64;
+  static constexpr int BM = NWAVES * 32;
+  static constexpr int K_PITCH = D * (QK8 ? 1 : 2);             // bytes per LDS row, no padding
+  static constexpr int V_PITCH = D * (PV8 ? 1 : 2);
+  static constexpr int K_TILE = BN * K_PITCH, V_TILE = BN * V_PITCH;
+  static constexpr int K_ST0 = 0, V_ST0 = 2 * K_TILE;           // LDS map: K stage 0/1, V stage 0/1
+  static constexpr int LDS_BYTES = 2 * K_TILE + 2 * V_TILE;
+  // one wave-wide 16 B/lane copy moves 1 KB = RPI rows; IPW copies per wave and tile
+  static constexpr int K_RPI = 1024 / K_PITCH, K_IPW = BN / K_RPI / NWAVES;
+  static constexpr int V_RPI = 1024 / V_PITCH, V_IPW = BN / V_RPI / NWAVES;
+  static_assert(D == 64 || D == 128 || D == 256, "head dim");
+  static_assert(BN % 32 == 0 && (!PV8 || BN == 64), "key tile: the e4m3 second GEMM has 64-deep K-steps");
+  static_assert(K_IPW >= 1 && K_IPW * K_RPI * NWAVES == BN && V_IPW >= 1 && V_IPW * V_RPI * NWAVES == BN,
+                "tile must split evenly over the waves");
+};
+
+// XOR swizzles of the 16-byte chunk index of an LDS row.  Banks repeat every 256 B, so 256/PITCH rows share a bank
+// period (PITCH <= 256) or a row spans several (PITCH = 512).
+//  rows read by ds_read_b128, 16 consecutive rows at one chunk index: rows at the same place in the bank period
+//  need distinct values.
+template <int PITCH>
+__device__ __forceinline__ int swz_row(int row) {
+  if (PITCH == 64) return (row >> 2) & 3;
+  if (PITCH == 128) return (row >> 1) & 7;
+  return ((row & 3) << 2) | ((row >> 2) & 3);
+}
+//  fp16 V read by ds_read_b64_tr_b16: 4 consecutive keys x 64 contiguous bytes.
+template <int PITCH>
+__device__ __forceinline__ int swz_v16(int row) {
+  if (PITCH == 128) return ((row >> 1) & 1) << 2;
+  return (row & 3) << 2;
+}
+//  e4m3 V read by ds_read_b64_tr_b8: keys {4g..4g+3, 8+4g..8+4g+3} x 32 contiguous bytes; bit 0 stays clear so a
+//  32-byte pair stays contiguous.
+template <int PITCH>
+__device__ __forceinline__ int swz_v8(int row) {
+  if (PITCH == 64) return ((row >> 3) & 1) << 1;
+  if (PITCH == 128) return (((row >> 1) & 1) << 1) | (((row >> 3) & 1) << 2);
+  return ((row & 3) | (((row >> 3) & 1) << 2)) << 1;
+}
+
+template <class C>
+__global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(C::WPE, C::WPE)))
+fmha_fwd_kernel(const FmhaArgs a) {
+  constexpr int D = C::D, BN = C::BN;
+  constexpr bool QK8 = C::QK8, PV8 = C::PV8;
+  constexpr int KB = BN / 32;                  // 32-key blocks per tile (M blocks of S^T)
+  constexpr int KS = QK8 ? D / 64 : D / 16;    // K-steps of S^T
+  constexpr int KH = QK8 ? 2 : 1;              // 16-byte LDS reads per K operand
+  constexpr int DB = D / 32;                   // 32-row blocks of O^T
+  constexpr int PS = PV8 ? BN / 64 : BN / 16;  // K-steps of O^T
+  constexpr float kTau = 8.0f;                 // deferred-rescale threshold (log2 domain)
+  constexpr float kPBias = PV8 ? 7.0f : 0.0f;  // the reference point sits this far below the row max
+  using QReg = std::conditional_t<QK8, int8v, half8>;
+  using PReg = std::conditional_t<PV8, int8v, half8>;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, g = lane >> 5;
+
+  const int q_blocks = a.Sq / C::BM;
+  const int tile = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = tile / q_blocks;
+  const int qb = tile - bh * q_blocks;
+  const int b = bh / a.H, h = bh - b * a.H;
+  const int64_t ld = (int64_t)a.H * D;  // row stride in elements
+  constexpr int QES = QK8 ? 1 : 2, VES = PV8 ? 1 : 2;
+  const char *Qp = (const char *)a.q + (((int64_t)b * a.Sq * a.H + h) * D) * QES;
+  const char *Kp = (const char *)a.k + (((int64_t)b * a.Skv * a.H + h) * D) * QES;
+  const char *Vp = (const char *)a.v + (((int64_t)b * a.Skv * a.H + h) * D) * VES;
+  _Float16 *Op = (_Float16 *)a.o + ((int64_t)b * a.Sq * a.H + h) * D;
+  const int q0 = qb * C::BM + wave * 32;
+  const int n_tiles = a.Skv / BN;
+  const float c_log2 = a.scale_log2;
+  const uint32_t k_ld = (uint32_t)(ld * QES), v_ld = (uint32_t)(ld * VES);  // global row pitch in bytes
+
+  // ---- global -> LDS copies.  Copy i of wave w covers tile rows (i*NWAVES + w)*RPI .. +RPI; lane l writes LDS slot
+  // (row l / CPR, chunk position l % CPR) and fetches chunk position ^ swz(row) of that row.
+  uint32_t goff_k[C::K_IPW], goff_v[C::V_IPW];
+#pragma unroll
+  for (int i = 0; i < C::K_IPW; ++i) {
+    constexpr int CPR = C::K_PITCH / 16;
+    const int row = (i * C::NWAVES + wave) * C::K_RPI + lane / CPR;
+    goff_k[i] = (uint32_t)row * k_ld + (uint32_t)(((lane % CPR) ^ swz_row<C::K_PITCH>(row)) * 16);
+  }
+#pragma unroll
+  for (int i = 0; i < C::V_IPW; ++i) {
+    constexpr int CPR = C::V_PITCH / 16;
+    const int row = (i * C::NWAVES + wave) * C::V_RPI + lane / CPR;
+    const int sw = PV8 ? swz_v8<C::V_PITCH>(row) : swz_v16<C::V_PITCH>(row);
+    goff_v[i] = (uint32_t)row * v_ld + (uint32_t)(((lane % CPR) ^ sw) * 16);
+  }
+  const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+  auto load_k = [&](int jt, int stage) {
+    const char *gt = Kp + (size_t)jt * ((size_t)BN * k_ld);
+#pragma unroll
+    for (int i = 0; i < C::K_IPW; ++i)
+      lds_dma16(gt + goff_k[i], lds_base + C::K_ST0 + stage * C::K_TILE + (i * C::NWAVES + wave) * 1024);
+  };
+  auto load_v = [&](int jt, int stage) {
+    const char *gt = Vp + (size_t)jt * ((size_t)BN * v_ld);
+#pragma unroll
+    for (int i = 0; i < C::V_IPW; ++i)
+      lds_dma16(gt + goff_v[i], lds_base + C::V_ST0 + stage * C::V_TILE + (i * C::NWAVES + wave) * 1024);
+  };
+
+  // ---- Q: B operand of S^T, resident in VGPRs.  fp16: lane (r, g), K-step s holds Q[q0+r][16s + 8g .. +8);
+  // e4m3: the 32 bytes Q[q0+r][64s + 32g .. +32) (which contraction slot means which d is free as long as the K
+  // operand uses the same map).
+  QReg qreg[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    if constexpr (QK8) {
+      const int4v *p = (const int4v *)(Qp + (int64_t)(q0 + r) * ld + 64 * s + 32 * g);
+      const int4v lo = p[0], hi = p[1];
+      qreg[s] = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    } else {
+      qreg[s] = *(const half8 *)(Qp + ((int64_t)(q0 + r) * ld + 16 * s + 8 * g) * 2);
+    }
+  }
+
+  // ---- per-lane LDS read addresses (bytes, relative to a tile)
+  // K operand, K-step s: row r (+32 kb); fp16 chunk 2s+g, e4m3 chunks 4s+2g and 4s+2g+1 (each swizzled on its own)
+  int k_rd[KS][KH];
+#pragma unroll
+  for (int s = 0; s < KS; ++s)
+#pragma unroll
+    for (int hh = 0; hh < KH; ++hh)
+      k_rd[s][hh] = r * C::K_PITCH + ((((QK8 ? 4 : 2) * s + KH * g + hh) ^ swz_row<C::K_PITCH>(r)) * 16);
+  // V operand: see the file comment.  li = lane within its block of 16.
+  const int li = lane & 15;
+  int v_rd[DB];
+  if constexpr (PV8) {
+    const int row_e = li >> 1;
+    const int v_key = 8 * (row_e >> 2) + 4 * g + (row_e & 3);  // + 16 u
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      v_rd[db] = v_key * C::V_PITCH + (((2 * db + ((lane >> 4) & 1)) ^ swz_v8<C::V_PITCH>(v_key)) * 16) + 8 * (li & 1);
+  } else {
+    const int v_key = 4 * g + (li >> 2);                       // + 16 ps + 8 h2
+    const int v_col = 16 * ((lane >> 4) & 1) + 4 * (li & 3);   // + 32 db   (element index)
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+      v_rd[db] = v_key * C::V_PITCH + ((((db * 32 + v_col) >> 3) ^ swz_v16<C::V_PITCH>(v_key)) * 16) + (v_col & 7) * 2;
+  }
+
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
+  float m_ref = -INFINITY, m_true = -INFINITY, l_run = 0.f;  // softmax reference point, true running max, running sum
+
+  // S^T = K . Q^T for the K tile in LDS stage `stage`
+  auto qk = [&](int stage, f32x16 (&sacc)[KB]) {
+    const char *kt = smem + C::K_ST0 + stage * C::K_TILE;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) sacc[kb][v] = 0.f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        if constexpr (QK8) {
+          const int4v lo = *(const int4v *)(kt + k_rd[s][0] + kb * 32 * C::K_PITCH);
+          const int4v hi = *(const int4v *)(kt + k_rd[s][1] + kb * 32 * C::K_PITCH);
+          const int8v ka = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka, qreg[s], sacc[kb], 0, 0, 0, 0, 0, 0);
+        } else {
+          const half8 ka = *(const half8 *)(kt + k_rd[s][0] + kb * 32 * C::K_PITCH);
+          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[s], sacc[kb], 0, 0, 0);
+        }
+      }
+  };
+  // Row max of a finished S tile and the deferred rescale (online_softmax.h:123-165).  The branch is wave-uniform.
+  auto row_max_and_rescale = [&](const f32x16 (&sacc)[KB]) {
+    float mx = sacc[0][0];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[kb][v]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * c_log2;
+    m_true = fmaxf(m_true, mx);
+    if (__builtin_amdgcn_ballot_w64(mx > m_ref + kTau) != 0) {
+      const float m_new = fmaxf(m_ref, mx - kPBias);
+      const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+      m_ref = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[db][v] *= alpha;
+    }
+  };
+  // P = exp2(c*S - m_ref); row sum in fp32 before the down-cast (online_softmax.h:173-206); cast in the B-operand
+  // register order of the second GEMM
+  auto softmax_exp = [&](const f32x16 (&sacc)[KB], PReg (&pb)[PS]) {
+    float rs = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        float p[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          p[t] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][4 * w + t], c_log2, -m_ref));
+          rs += p[t];
+        }
+        if constexpr (PV8) {  // slot 16 kb + 4 w + t
+          int packed = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+          pb[kb / 2][(kb % 2) * 4 + w] = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], packed, true);
+        } else {              // K-step 2 kb + w / 2, slot 4 (w % 2) + t
+#pragma unroll
+          for (int t = 0; t < 4; ++t) pb[kb * 2 + w / 2][4 * (w % 2) + t] = (_Float16)p[t];
+        }
+      }
+    l_run += rs;
+  };
+  // O^T += V^T . P^T for the V tile in LDS stage `stage`
+  auto pv = [&](int stage, const PReg (&pb)[PS]) {
+    const char *vt = smem + C::V_ST0 + stage * C::V_TILE;
+#pragma unroll
+    for (int ps = 0; ps < PS; ++ps)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        if constexpr (PV8) {
+          int8v va;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int2v x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(int2v, vt + v_rd[db] + (ps * 64 + u * 16) * C::V_PITCH));
+            va[2 * u] = x[0];
+            va[2 * u + 1] = x[1];
+          }
+          oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb[ps], oacc[db], 0, 0, 0, 0, 0, 0);
+        } else {
+          const char *vp = vt + v_rd[db] + ps * 16 * C::V_PITCH;
+          union {
+            struct { short4v lo, hi; } s;
+            half8 h;
+          } va;
+          va.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, vp));
+          va.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, vp + 8 * C::V_PITCH));
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va.h, pb[ps], oacc[db], 0, 0, 0);
+        }
+      }
+  };
+
+  // One pipeline step for tile j (parity P = j & 1).  On entry: s_cur = S_j is finished and its max is folded into
+  // m_ref; K_{j+1} sits in K stage P^1 and V_j in V stage P.  HAS_NEXT is false for the last tile only.
+  auto step = [&](auto parity, auto has_next, int j, f32x16 (&s_cur)[KB], f32x16 (&s_nxt)[KB]) {
+    constexpr int P = decltype(parity)::value;
+    constexpr bool HAS_NEXT = decltype(has_next)::value;
+    // prefetch K_{j+2} into K stage P (last read by step j-1) and V_{j+1} into V stage P^1 (ditto); the indices are
+    // clamped at the end, which only rewrites a stage nobody reads any more
+    load_k(j + 2 < n_tiles ? j + 2 : n_tiles - 1, P);
+    load_v(j + 1 < n_tiles ? j + 1 : n_tiles - 1, P ^ 1);
+    PReg pb[PS];
+    if (HAS_NEXT) qk(P ^ 1, s_nxt);
+    softmax_exp(s_cur, pb);
+    pv(P, pb);
+    if (HAS_NEXT) row_max_and_rescale(s_nxt);
+    wait_lds_dma();   // this wave's copies have landed ...
+    __syncthreads();  // ... and so have everybody else's; all reads of the stages about to be refilled are done
+  };
+
+  // ---- prologue: K_0, V_0, K_1 in flight; S_0 and its row max
+  f32x16 s_a[KB], s_b[KB];
+  load_k(0, 0);
+  load_v(0, 0);
+  load_k(n_tiles > 1 ? 1 : 0, 1);
+  wait_lds_dma();
+  __syncthreads();
+  qk(0, s_a);
+  row_max_and_rescale(s_a);
+  __syncthreads();  // every wave is done with K stage 0 before step 0 overwrites it
+
+  using std::integral_constant;
+  int j = 0;
+  for (; j + 2 < n_tiles; j += 2) {
+    step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
+    step(integral_constant<int, 1>{}, integral_constant<bool, true>{}, j + 1, s_b, s_a);
+  }
+  if (j + 2 == n_tiles) {  // two tiles left: j (even) with a successor, then the last one
+    step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
+    step(integral_constant<int, 1>{}, integral_constant<bool, false>{}, j + 1, s_b, s_a);
+  } else {                 // one tile left (even index)
+    step(integral_constant<int, 0>{}, integral_constant<bool, false>{}, j, s_a, s_b);
+  }
+
+  // ---- epilogue: O = out_scale * O / l (online_softmax.h:59-85), fp16, [B,S,H,D]; a lane holds 4 consecutive d
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv = a.out_scale / l_tot;
+  const int qrow = q0 + r;
+  _Float16 *orow = Op + (int64_t)qrow * ld;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      half4 o4;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) o4[t] = (_Float16)(oacc[db][4 * i + t] * inv);
+      *(half4 *)(orow + db * 32 + 8 * i + 4 * g) = o4;
+    }
+  if (g == 0) {
+    const int64_t si = ((int64_t)b * a.H + h) * a.Sq + qrow;
+    // taps are reported against the true row max, as the reference's miOut / sPrimeOut are (fmha_epilogue.h:7-46)
+    if (a.row_max) a.row_max[si] = m_true;
+    if (a.row_sum) a.row_sum[si] = l_tot * __builtin_amdgcn_exp2f(m_ref - m_true);
+  }
+}
+
+template <class C>
+hipError_t launch_fmha_cfg(const FmhaArgs &a, hipStream_t s) {
+  static bool attr_done = false;  // one attribute call per instantiation and process
+  auto kern = fmha_fwd_kernel<C>;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    attr_done = true;
+  }
+  const int grid = a.B * a.H * (a.Sq / C::BM);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::T), C::LDS_BYTES, s, a);
+  return hipGetLastError();
+}
+
+template <class C>
+void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
+  p->block_m = C::BM;
+  p->block_n = C::BN;
+  p->lds_bytes = C::LDS_BYTES;
+  p->threads = C::T;
+  p->grid = bh * (sq / C::BM);
+}
+
+// CFK_FMHA_TILE=small|large forces the 128-row or the 256-row workgroup tile where both exist (tuning aid; the
+// reference picks its tile with -DQBLKSIZE/-DKBLKSIZE at compile time, src/fmha-pipeline/shared_storage.h:4-15).
+// Otherwise the large tile is used where it measured faster (`prefer_large`: the fp16-P paths) when
+// seqlen_q % 256 == 0 and there are enough workgroups to fill 256 CUs twice.
+inline bool use_large_tile(int sq, int bh, bool prefer_large = true) {
+  static const int forced = [] {
+    const char *e = getenv("CFK_FMHA_TILE");
+    if (!e) return -1;
+    return e[0] == 's' ? 0 : e[0] == 'l' ? 1 : -1;
+  }();
+  if (sq % 256 != 0 || forced == 0) return false;
+  if (forced == 1) return true;
+  return prefer_large && (long long)bh * (sq / 256) >= 512;
+}
+
+}  // namespace cfk

@@ -22,13 +22,6 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 
-#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T *)(p))
-
-__device__ __forceinline__ void lds_dma16(const void *gptr, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
-}
-__device__ __forceinline__ void wait_lds_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
 constexpr int BM = 256, BN = 256, BK = 64, NWAVES = 8, T = NWAVES * 64;
 constexpr int A_TILE = BM * BK * 2;            // 32 KB, rows of 128 B (K-contiguous)
 constexpr int B_TILE = BN * BK * 2;            // 32 KB: TN rows of 128 B (n rows); NN rows of 512 B (k rows)

@@ -8,6 +8,8 @@
 // plus, not in the reference:
 //   --fp8-scales=unit|amax   unit (default) casts N(0,1) straight to e4m3 as the reference does (:498-500);
 //                            amax applies per-tensor amax/448 scales and passes the descales to the library
+//   --gemm2-fp8=true         with --prec-type=2: true = P and V in e4m3 too (the reference built with -DGEMM2FP8),
+//                            false = hybrid, Q,K e4m3 with fp16 P,V (the reference's default build, :446-450)
 //   --verify-all=false       also checks the row-max / row-sum taps (the reference's -DCOPYOUTMI build, :655-676)
 //   --dump-dir=<dir>         writes q.bin k.bin v.bin o.bin (+ meta.txt) for an external checker
 //
@@ -41,6 +43,7 @@ namespace {
 
 struct Options {
   int batch = 4, dim = 2048, head = 64, seq = 4096, iterations = 20, streams = 1, prec = 2;
+  bool gemm2_fp8 = true;
   bool ref_check = false, print_values = false, print_diffs = false, verify_all = false, help = false, selftest = false;
   std::string fp8_scales = "unit", dump_dir;
 };
@@ -67,6 +70,7 @@ bool parse(int argc, char **argv, Options &o) {
     else if (key == "prec-type") o.prec = atoi(val);
     else if (key == "fp8-scales") o.fp8_scales = val;
     else if (key == "verify-all") o.verify_all = parse_bool(val);
+    else if (key == "gemm2-fp8") o.gemm2_fp8 = parse_bool(val);
     else if (key == "dump-dir") o.dump_dir = val;
     else if (key == "selftest-e4m3") o.selftest = true;
     else return false;
@@ -89,6 +93,7 @@ void print_usage() {
       "  --print-values=<bool>       If true, prints the values of the result.\n"
       "  --print-diffs=<bool>        If true, prints every element that fails the check.\n"
       "  --fp8-scales=unit|amax      fp8 quantisation: unit scales (reference behaviour) or per-tensor amax.\n"
+      "  --gemm2-fp8=<bool>          fp8 only: P and V in e4m3 too (default true); false = fp16 P and V.\n"
       "  --verify-all=<bool>         Also check the row-max / row-sum taps.\n"
       "  --dump-dir=<dir>            Write q.bin k.bin v.bin o.bin meta.txt there.\n");
 }
@@ -232,10 +237,12 @@ int main(int argc, char **argv) {
   }
   const int B = opt.batch, S = opt.seq, D = opt.head, H = opt.dim / opt.head;
   const bool fp8 = opt.prec == 2;
+  const bool v_fp8 = fp8 && opt.gemm2_fp8;
   const float softmax_scale = 1.0f / std::sqrt((float)D);
 
   cfk_fmha_fwd_params plan_q{};
-  plan_q.dtype = plan_q.v_dtype = opt.prec;
+  plan_q.dtype = opt.prec;
+  plan_q.v_dtype = v_fp8 ? CFK_FP8_E4M3 : CFK_FP16;
   plan_q.batch = B / opt.streams;
   plan_q.heads = H;
   plan_q.seqlen_q = plan_q.seqlen_kv = S;
@@ -259,14 +266,14 @@ int main(int argc, char **argv) {
     for (size_t i = 0; i < n; ++i) hk[i] = nd(g2);
     for (size_t i = 0; i < n; ++i) hv[i] = nd(g3);
   }
-  const size_t esz = fp8 ? 1 : 2;
-  std::vector<uint8_t> qb(n * esz), kb(n * esz), vb(n * esz);
+  const size_t esz = fp8 ? 1 : 2, vesz = v_fp8 ? 1 : 2;
+  std::vector<uint8_t> qb(n * esz), kb(n * esz), vb(n * vesz);
   float descale[3] = {1.f, 1.f, 1.f};
   std::vector<float> *src[3] = {&hq, &hk, &hv};
   std::vector<uint8_t> *dst[3] = {&qb, &kb, &vb};
   for (int t = 0; t < 3; ++t) {
     std::vector<float> &x = *src[t];
-    if (fp8) {
+    if (t == 2 ? v_fp8 : fp8) {
       if (opt.fp8_scales == "amax") {
         float amax = 0.f;
         for (float v : x) amax = std::fmax(amax, std::fabs(v));
@@ -290,13 +297,13 @@ int main(int argc, char **argv) {
   float *dmi, *dsp;
   HIP_CHECK(hipMalloc(&dq, n * esz));
   HIP_CHECK(hipMalloc(&dk, n * esz));
-  HIP_CHECK(hipMalloc(&dv, n * esz));
+  HIP_CHECK(hipMalloc(&dv, n * vesz));
   HIP_CHECK(hipMalloc(&dout, n * 2));
   HIP_CHECK(hipMalloc(&dmi, (size_t)B * H * S * 4));
   HIP_CHECK(hipMalloc(&dsp, (size_t)B * H * S * 4));
   HIP_CHECK(hipMemcpy(dq, qb.data(), n * esz, hipMemcpyHostToDevice));
   HIP_CHECK(hipMemcpy(dk, kb.data(), n * esz, hipMemcpyHostToDevice));
-  HIP_CHECK(hipMemcpy(dv, vb.data(), n * esz, hipMemcpyHostToDevice));
+  HIP_CHECK(hipMemcpy(dv, vb.data(), n * vesz, hipMemcpyHostToDevice));
   {  // O is pre-filled with -1 (fmha_forward.cu:501-502)
     std::vector<_Float16> neg(n, (_Float16)-1.0f);
     HIP_CHECK(hipMemcpy(dout, neg.data(), n * 2, hipMemcpyHostToDevice));
@@ -314,7 +321,7 @@ int main(int argc, char **argv) {
         const size_t off = (size_t)i * Lb * S * H * D;
         p.q = (const char *)dq + off * esz;
         p.k = (const char *)dk + off * esz;
-        p.v = (const char *)dv + off * esz;
+        p.v = (const char *)dv + off * vesz;
         p.o = (char *)dout + off * 2;
         p.q_descale = descale[0];
         p.k_descale = descale[1];
@@ -357,8 +364,8 @@ int main(int argc, char **argv) {
     bool ok = write_file(opt.dump_dir + "/q.bin", qb.data(), qb.size()) && write_file(opt.dump_dir + "/k.bin", kb.data(), kb.size()) &&
               write_file(opt.dump_dir + "/v.bin", vb.data(), vb.size()) && write_file(opt.dump_dir + "/o.bin", ho.data(), n * 2);
     char meta[512];
-    snprintf(meta, sizeof(meta), "prec %d\nB %d\nS %d\nH %d\nD %d\nq_descale %.9g\nk_descale %.9g\nv_descale %.9g\nsoftmax_scale %.9g\n",
-             opt.prec, B, S, H, D, descale[0], descale[1], descale[2], softmax_scale);
+    snprintf(meta, sizeof(meta), "prec %d\nv_fp8 %d\nB %d\nS %d\nH %d\nD %d\nq_descale %.9g\nk_descale %.9g\nv_descale %.9g\nsoftmax_scale %.9g\n",
+             opt.prec, (int)v_fp8, B, S, H, D, descale[0], descale[1], descale[2], softmax_scale);
     ok = ok && write_file(opt.dump_dir + "/meta.txt", meta, strlen(meta));
     if (!ok) {
       fprintf(stderr, "could not write to %s\n", opt.dump_dir.c_str());

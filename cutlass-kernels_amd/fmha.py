@@ -125,7 +125,8 @@ def fmha_forward(q, k, v, o=None, softmax_scale=None, q_descale=1.0, k_descale=1
                  v_layout=CFK_V_BSHD, row_max=None, row_sum=None, stream=None):
     """O = softmax(scale * Q K^T) V on device tensors in [B,S,H,D] (D contiguous).
 
-    q,k,v: torch CUDA tensors, float16, or float8_e4m3fn / uint8 holding e4m3 codes.  ``v`` is [B,D,H,S] when
+    q,k,v: torch CUDA tensors, float16, or float8_e4m3fn / uint8 holding e4m3 codes (v may be float16 with e4m3
+    q,k: hybrid mode).  ``v`` is [B,D,H,S] when
     ``v_layout == CFK_V_BDHS``.  Returns ``o`` (float16 [B,Sq,H,D]); launches asynchronously on ``stream``
     (default: torch's current stream)."""
     import torch
@@ -139,8 +140,14 @@ def fmha_forward(q, k, v, o=None, softmax_scale=None, q_descale=1.0, k_descale=1
         dtype = CFK_FP8_E4M3
     else:
         raise ValueError(f"unsupported dtype {q.dtype}")
-    if k.dtype != q.dtype or v.dtype != q.dtype:
-        raise ValueError("q, k, v must share one dtype")
+    if k.dtype != q.dtype:
+        raise ValueError("q and k must share one dtype")
+    if v.dtype == q.dtype:
+        v_dtype = dtype
+    elif dtype == CFK_FP8_E4M3 and v.dtype == torch.float16:
+        v_dtype = CFK_FP16  # hybrid mode: e4m3 Q,K with fp16 P,V (the reference's fp8 build without GEMM2FP8)
+    else:
+        raise ValueError("v must have the dtype of q, or float16 with fp8 q/k")
     B, Sq, H, D = q.shape
     Skv = k.shape[1]
     if tuple(k.shape) != (B, Skv, H, D):
@@ -156,7 +163,7 @@ def fmha_forward(q, k, v, o=None, softmax_scale=None, q_descale=1.0, k_descale=1
         if t is not None and (t.dtype != torch.float32 or tuple(t.shape) != (B, H, Sq) or not t.is_contiguous()):
             raise ValueError("row_max/row_sum must be contiguous float32 [B,H,Sq]")
     p = make_params(dtype, B, H, Sq, Skv, D, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), softmax_scale,
-                    q_descale, k_descale, v_descale, v_layout,
+                    q_descale, k_descale, v_descale, v_layout, v_dtype=v_dtype,
                     dbg_row_max=row_max.data_ptr() if row_max is not None else 0,
                     dbg_row_sum=row_sum.data_ptr() if row_sum is not None else 0)
     _check(lib().cfk_fmha_forward(ctypes.byref(p), _stream_ptr(stream)))

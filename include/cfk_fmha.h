@@ -50,8 +50,9 @@ typedef enum cfk_v_layout {
  */
 typedef struct cfk_fmha_fwd_params {
   int32_t dtype;     /* cfk_dtype of Q and K                                                                  */
-  int32_t v_dtype;   /* cfk_dtype of V (and of P): must equal dtype; CFK_FP16 with dtype = CFK_FP8_E4M3 is the
-                        reference's hybrid mode (fmha_forward.cu:446-450) and is reported CFK_ERR_UNSUPPORTED */
+  int32_t v_dtype;   /* cfk_dtype of V (and of P).  Equal to dtype, or CFK_FP16 with dtype = CFK_FP8_E4M3: the
+                        reference's hybrid mode, fp8 Q,K with fp16 P,V -- what its --prec-type=2 computes when built
+                        without -DGEMM2FP8 (fmha_forward.cu:446-450)                                            */
   int32_t batch;     /* BATCH                                                                                 */
   int32_t heads;     /* NUMHEADS                                                                              */
   int32_t seqlen_q;  /* SEQLEN: multiple of 128                                                               */
@@ -66,7 +67,7 @@ typedef struct cfk_fmha_fwd_params {
                           (The reference passes scale*log2e, fmha_forward.cu:452-454.)                        */
   float q_descale;   /* fp8 per-tensor scales: real value = code value * descale.  1.0f reproduces the        */
   float k_descale;   /* reference, which applies no scaling (fmha_forward.cu:498-500).  Ignored for fp16.     */
-  float v_descale;
+  float v_descale;   /* ignored when v_dtype is CFK_FP16                                                      */
   float *dbg_row_max; /* optional tap, [B, H, S_q] fp32: running row max in the log2 domain (score*scale*log2e),
                          the reference's miOut under COPYOUTMI (fmha_epilogue.h:7-46); NULL = off              */
   float *dbg_row_sum; /* optional tap, [B, H, S_q] fp32: row sum of exp2(t - max), not its reciprocal, the

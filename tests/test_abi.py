@@ -36,6 +36,7 @@ def test_version_and_plan_without_gpu():
     assert 2048 % bm == 0 and 2048 % bn == 0 and 0 < lds <= 160 * 1024 and threads % 64 == 0
     for d in (64, 128, 256):
         pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, d)
+        pkg.fmha_forward_plan(pkg.CFK_FP8_E4M3, 1, 1, 512, 512, d)
 
 
 def test_error_paths_mirror_reference_driver():
@@ -52,8 +53,9 @@ def test_error_paths_mirror_reference_driver():
     with pytest.raises(pkg.CfkError) as e:
         pkg.fmha_forward_plan(pkg.CFK_FP16, 0, 1, 512, 512, 64)
     assert e.value.code == -1
+    pkg.fmha_forward_plan(pkg.CFK_FP8_E4M3, 1, 1, 512, 512, 64, v_dtype=pkg.CFK_FP16)      # hybrid mode
     with pytest.raises(pkg.CfkError):
-        pkg.fmha_forward_plan(pkg.CFK_FP8_E4M3, 1, 1, 512, 512, 64, v_dtype=pkg.CFK_FP16)  # hybrid mode not built
+        pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, 64, v_dtype=pkg.CFK_FP8_E4M3)  # not a reference mode
     with pytest.raises(pkg.CfkError):
         pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, 64, v_layout=1)
     # null params / null pointers

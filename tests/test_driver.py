@@ -52,15 +52,20 @@ def _load_dump(d):
         q, k, v = (np.fromfile(os.path.join(d, f + ".bin"), dtype=np.float16).reshape(shape).astype(np.float32)
                    for f in "qkv")
     else:
-        q, k, v = (oracle.e4m3_decode(np.fromfile(os.path.join(d, f + ".bin"), dtype=np.uint8).reshape(shape)) *
-                   np.float32(meta[f + "_descale"]) for f in "qkv")
+        q, k = (oracle.e4m3_decode(np.fromfile(os.path.join(d, f + ".bin"), dtype=np.uint8).reshape(shape)) *
+                np.float32(meta[f + "_descale"]) for f in "qk")
+        if int(meta["v_fp8"]):
+            v = oracle.e4m3_decode(np.fromfile(os.path.join(d, "v.bin"), dtype=np.uint8).reshape(shape)) * \
+                np.float32(meta["v_descale"])
+        else:
+            v = np.fromfile(os.path.join(d, "v.bin"), dtype=np.float16).reshape(shape).astype(np.float32)
     o = np.fromfile(os.path.join(d, "o.bin"), dtype=np.float16).reshape(shape).astype(np.float32)
     return q, k, v, o, prec
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("prec,head,extra", [(1, 64, []), (1, 128, ["--num-cuda-streams=2"]), (1, 256, []),
-                                             (2, 128, []), (2, 128, ["--fp8-scales=amax"]), (2, 64, []), (2, 256, [])])
+                                             (2, 128, []), (2, 128, ["--fp8-scales=amax"]), (2, 64, []), (2, 256, []), (2, 128, ["--gemm2-fp8=false"])])
 def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
     # fp8 needs the reference's own sequence length for its percentage criterion; fp16 passes at any length
     seq = 2048 if prec == 2 else 512

@@ -118,6 +118,41 @@ def test_taps_and_invariants():
     np.testing.assert_allclose(sel[0, :, 0], np.broadcast_to(vf2[0, 77, 0], sel[0, :, 0].shape), rtol=2e-3, atol=1e-4)  # fp16 output rounding only
 
 
+@pytest.mark.parametrize("B,S,H,D", [(1, 512, 2, 128), (2, 256, 3, 64), (1, 384, 2, 256), (2, 2048, 4, 128)])
+def test_hybrid_mode_fp8_qk_fp16_pv(B, S, H, D):
+    # the reference's --prec-type=2 without -DGEMM2FP8: Q,K e4m3, P and V fp16 (fmha_forward.cu:446-450).
+    # GEMM-I on e4m3 products is exact in fp32, so the error is that of the fp16 path.
+    import torch
+    from _util import ERRPCT_FP16, TOL_FP16
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    (qc, qs, qf), (kc, ks, kf) = _quant(q), _quant(k)
+    v16 = v.astype(np.float16)
+    o = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(v16), q_descale=qs, k_descale=ks)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    ref = oracle.attention_f32(qf, kf, v16.astype(np.float32))["O"]
+    err = max_abs(got, ref)
+    ok, pct = oracle.verify_tensor(got, ref, ERRPCT_FP16)
+    print(f"hybrid B={B} S={S} H={H} D={D}: max-abs {err:.3e}, error% {pct:.2e}")
+    assert err <= TOL_FP16 and ok
+
+
+def test_hybrid_exact_arithmetic():
+    rng = np.random.default_rng(12)
+    for D in (64, 128, 256):
+        B, S, H = 1, 384, 2
+        q = np.zeros((B, S, H, D), np.float32)
+        np.put_along_axis(q, rng.integers(0, D, (B, S, H, 4)), 1.0, axis=-1)
+        k = rng.integers(-1, 2, (B, S, H, D)).astype(np.float32)
+        v = rng.integers(-8, 9, (B, S, H, D)).astype(np.float32)
+        import torch
+        o = pkg.fmha_forward(to_dev(oracle.e4m3_encode(q)), to_dev(oracle.e4m3_encode(k)), to_dev(v.astype(np.float16)),
+                             softmax_scale=float(np.log(2.0)))
+        torch.cuda.synchronize()
+        ref = oracle.attention_f32(q, k, v, alpha0=np.log(2.0))["O"]
+        np.testing.assert_allclose(o.float().cpu().numpy(), ref, rtol=1.5e-3, atol=2e-4)
+
+
 def test_unsupported_modes_report_errors():
     import torch
     x = torch.zeros((1, 128, 1, 64), dtype=torch.uint8, device="cuda:0")
