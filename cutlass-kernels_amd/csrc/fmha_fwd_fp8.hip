@@ -10,8 +10,21 @@ using Cfg128S = FmhaCfg<128, 64, 4, 2, true, true>;
 using Cfg128L = FmhaCfg<128, 64, 8, 2, true, true>;
 using Cfg256S = FmhaCfg<256, 64, 4, 1, true, true>;  // O (128) + S (64) + Q (32) registers: one wave per SIMD
 
+// V pre-transposed to [B,D,H,S] (the reference's offline transpose, src/fmha-pipeline/fmha_forward.cu:514-532)
+using Cfg64T = FmhaCfg<64, 64, 4, 2, true, true, true>;
+using Cfg128T = FmhaCfg<128, 64, 4, 2, true, true, true>;
+using Cfg256T = FmhaCfg<256, 64, 4, 1, true, true, true>;
+
 template <class F>
-bool dispatch(int head_dim, int sq, int bh, F &&f) {
+bool dispatch(int head_dim, int sq, int bh, int v_layout, F &&f) {
+  if (v_layout == 1) {
+    switch (head_dim) {
+      case 64: f(Cfg64T{}); return true;
+      case 128: f(Cfg128T{}); return true;
+      case 256: f(Cfg256T{}); return true;
+      default: return false;
+    }
+  }
   switch (head_dim) {
     case 64: f(Cfg64S{}); return true;
     case 128: use_large_tile(sq, bh, false) ? f(Cfg128L{}) : f(Cfg128S{}); return true;
@@ -24,14 +37,12 @@ bool dispatch(int head_dim, int sq, int bh, F &&f) {
 
 bool plan_fmha_fp8(int head_dim, int sq, int skv, int bh, int v_layout, FmhaPlan *p) {
   (void)skv;
-  if (v_layout != 0) return false;
-  return dispatch(head_dim, sq, bh, [&](auto cfg) { fill_fmha_plan<decltype(cfg)>(sq, bh, p); });
+  return dispatch(head_dim, sq, bh, v_layout, [&](auto cfg) { fill_fmha_plan<decltype(cfg)>(sq, bh, p); });
 }
 
 hipError_t launch_fmha_fp8(const FmhaArgs &a, int head_dim, hipStream_t s) {
-  if (a.v_layout != 0) return hipErrorNotSupported;
   hipError_t e = hipErrorNotSupported;
-  dispatch(head_dim, a.Sq, a.B * a.H, [&](auto cfg) { e = launch_fmha_cfg<decltype(cfg)>(a, s); });
+  dispatch(head_dim, a.Sq, a.B * a.H, a.v_layout, [&](auto cfg) { e = launch_fmha_cfg<decltype(cfg)>(a, s); });
   return e;
 }
 

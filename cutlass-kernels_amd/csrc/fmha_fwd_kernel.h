@@ -43,6 +43,10 @@
 //    e4m3).  With e4m3 P the reference point additionally sits 7 below the row max, so P spans (0, 2^8] instead of
 //    (0, 1] and probabilities down to 2^-17 of the row max stay out of e4m3's flush zone (the reference casts P in
 //    (0,1] directly, fmha_consumer.h:54); the bias cancels in O/l.
+//      - e4m3 V given pre-transposed [B,D,H,S] (the reference's offline transpose): the tile is [d][key]; the K
+//        tile is loaded row-permuted instead so that a lane's P slots are 32 contiguous keys and the V^T operand
+//        is two plain ds_read_b128 (the counterpart of the reference's FP8NOSHFL key permutation, done on K, in
+//        the copy, at no cost).
 //  * Per-tensor fp8 scales: q_descale*k_descale is folded into the exp2 scale, v_descale into the final 1/l.
 //  * Workgroup ids are remapped so the query blocks of one head share an XCD's L2.
 #pragma once
@@ -60,24 +64,27 @@ typedef int int8v __attribute__((ext_vector_type(8)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int2v __attribute__((ext_vector_type(2)));
 
-template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_>
+template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_, bool VT_ = false>
 struct FmhaCfg {
   static constexpr int D = D_, BN = BN_, NWAVES = NWAVES_;
   static constexpr int WPE = WPE_;                              // waves per SIMD the register budget is sized for
   static constexpr bool QK8 = QK8_, PV8 = PV8_;                 // e4m3 (true) or fp16 (false) operands of GEMM-I / II
+  static constexpr bool VT = VT_;                               // V given pre-transposed, [B,D,H,S] (e4m3 only)
   static constexpr int T = NWAVES * 64;
   static constexpr int BM = NWAVES * 32;
   static constexpr int K_PITCH = D * (QK8 ? 1 : 2);             // bytes per LDS row, no padding
-  static constexpr int V_PITCH = D * (PV8 ? 1 : 2);
-  static constexpr int K_TILE = BN * K_PITCH, V_TILE = BN * V_PITCH;
+  static constexpr int V_PITCH = VT ? BN : D * (PV8 ? 1 : 2);   // VT: the tile is [d][key], rows of BN bytes
+  static constexpr int V_ROWS = VT ? D : BN;
+  static constexpr int K_TILE = BN * K_PITCH, V_TILE = V_ROWS * V_PITCH;
   static constexpr int K_ST0 = 0, V_ST0 = 2 * K_TILE;           // LDS map: K stage 0/1, V stage 0/1
   static constexpr int LDS_BYTES = 2 * K_TILE + 2 * V_TILE;
   // one wave-wide 16 B/lane copy moves 1 KB = RPI rows; IPW copies per wave and tile
   static constexpr int K_RPI = 1024 / K_PITCH, K_IPW = BN / K_RPI / NWAVES;
-  static constexpr int V_RPI = 1024 / V_PITCH, V_IPW = BN / V_RPI / NWAVES;
+  static constexpr int V_RPI = 1024 / V_PITCH, V_IPW = V_ROWS / V_RPI / NWAVES;
   static_assert(D == 64 || D == 128 || D == 256, "head dim");
   static_assert(BN % 32 == 0 && (!PV8 || BN == 64), "key tile: the e4m3 second GEMM has 64-deep K-steps");
-  static_assert(K_IPW >= 1 && K_IPW * K_RPI * NWAVES == BN && V_IPW >= 1 && V_IPW * V_RPI * NWAVES == BN,
+  static_assert(!VT || PV8, "the pre-transposed layout is an e4m3-V layout");
+  static_assert(K_IPW >= 1 && K_IPW * K_RPI * NWAVES == BN && V_IPW >= 1 && V_IPW * V_RPI * NWAVES == V_ROWS,
                 "tile must split evenly over the waves");
 };
 
@@ -136,12 +143,15 @@ fmha_fwd_kernel(const FmhaArgs a) {
   constexpr int QES = QK8 ? 1 : 2, VES = PV8 ? 1 : 2;
   const char *Qp = (const char *)a.q + (((int64_t)b * a.Sq * a.H + h) * D) * QES;
   const char *Kp = (const char *)a.k + (((int64_t)b * a.Skv * a.H + h) * D) * QES;
-  const char *Vp = (const char *)a.v + (((int64_t)b * a.Skv * a.H + h) * D) * VES;
+  // V: [B,S,H,D] rows of the head at pitch H*D; pre-transposed [B,D,H,S]: rows d of the head at pitch H*Skv
+  const char *Vp = C::VT ? (const char *)a.v + ((int64_t)b * D * a.H + h) * a.Skv
+                         : (const char *)a.v + (((int64_t)b * a.Skv * a.H + h) * D) * VES;
   _Float16 *Op = (_Float16 *)a.o + ((int64_t)b * a.Sq * a.H + h) * D;
   const int q0 = qb * C::BM + wave * 32;
   const int n_tiles = a.Skv / BN;
   const float c_log2 = a.scale_log2;
-  const uint32_t k_ld = (uint32_t)(ld * QES), v_ld = (uint32_t)(ld * VES);  // global row pitch in bytes
+  // global row pitch in bytes
+  const uint32_t k_ld = (uint32_t)(ld * QES), v_ld = C::VT ? (uint32_t)a.H * (uint32_t)a.Skv : (uint32_t)(ld * VES);
 
   // ---- global -> LDS copies.  Copy i of wave w covers tile rows (i*NWAVES + w)*RPI .. +RPI; lane l writes LDS slot
   // (row l / CPR, chunk position l % CPR) and fetches chunk position ^ swz(row) of that row.
@@ -150,13 +160,17 @@ fmha_fwd_kernel(const FmhaArgs a) {
   for (int i = 0; i < C::K_IPW; ++i) {
     constexpr int CPR = C::K_PITCH / 16;
     const int row = (i * C::NWAVES + wave) * C::K_RPI + lane / CPR;
-    goff_k[i] = (uint32_t)row * k_ld + (uint32_t)(((lane % CPR) ^ swz_row<C::K_PITCH>(row)) * 16);
+    // Pre-transposed V wants a lane's 32 P slots to be 32 CONTIGUOUS keys.  Which key sits in which MFMA row of
+    // S^T is free, so the K tile is loaded row-permuted: LDS row 32kb + 8w + 4g + j holds key 32g + 16kb + 4w + j
+    // (then slot t of lane half g is key 32g + t).
+    const int key = C::VT ? 32 * ((row >> 2) & 1) + 16 * (row >> 5) + 4 * ((row >> 3) & 3) + (row & 3) : row;
+    goff_k[i] = (uint32_t)key * k_ld + (uint32_t)(((lane % CPR) ^ swz_row<C::K_PITCH>(row)) * 16);
   }
 #pragma unroll
   for (int i = 0; i < C::V_IPW; ++i) {
     constexpr int CPR = C::V_PITCH / 16;
     const int row = (i * C::NWAVES + wave) * C::V_RPI + lane / CPR;
-    const int sw = PV8 ? swz_v8<C::V_PITCH>(row) : swz_v16<C::V_PITCH>(row);
+    const int sw = C::VT ? swz_row<C::V_PITCH>(row) : PV8 ? swz_v8<C::V_PITCH>(row) : swz_v16<C::V_PITCH>(row);
     goff_v[i] = (uint32_t)row * v_ld + (uint32_t)(((lane % CPR) ^ sw) * 16);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
@@ -167,7 +181,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
       lds_dma16(gt + goff_k[i], lds_base + C::K_ST0 + stage * C::K_TILE + (i * C::NWAVES + wave) * 1024);
   };
   auto load_v = [&](int jt, int stage) {
-    const char *gt = Vp + (size_t)jt * ((size_t)BN * v_ld);
+    const char *gt = C::VT ? Vp + (size_t)jt * BN : Vp + (size_t)jt * ((size_t)BN * v_ld);
 #pragma unroll
     for (int i = 0; i < C::V_IPW; ++i)
       lds_dma16(gt + goff_v[i], lds_base + C::V_ST0 + stage * C::V_TILE + (i * C::NWAVES + wave) * 1024);
@@ -199,7 +213,13 @@ fmha_fwd_kernel(const FmhaArgs a) {
   // V operand: see the file comment.  li = lane within its block of 16.
   const int li = lane & 15;
   int v_rd[DB];
-  if constexpr (PV8) {
+  int vt_rd[2] = {0, 0};
+  if constexpr (C::VT) {  // row d = 32db + r of the [d][key] tile, chunks 2g and 2g+1 = keys 32g .. 32g+31
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) vt_rd[hh] = r * C::V_PITCH + (((2 * g + hh) ^ swz_row<C::V_PITCH>(r)) * 16);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) v_rd[db] = 0;
+  } else if constexpr (PV8) {
     const int row_e = li >> 1;
     const int v_key = 8 * (row_e >> 2) + 4 * g + (row_e & 3);  // + 16 u
 #pragma unroll
@@ -293,7 +313,12 @@ fmha_fwd_kernel(const FmhaArgs a) {
     for (int ps = 0; ps < PS; ++ps)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        if constexpr (PV8) {
+        if constexpr (C::VT) {
+          const int4v lo = *(const int4v *)(vt + vt_rd[0] + db * 32 * C::V_PITCH);
+          const int4v hi = *(const int4v *)(vt + vt_rd[1] + db * 32 * C::V_PITCH);
+          const int8v va = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb[ps], oacc[db], 0, 0, 0, 0, 0, 0);
+        } else if constexpr (PV8) {
           int8v va;
 #pragma unroll
           for (int u = 0; u < 4; ++u) {

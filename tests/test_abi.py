@@ -58,6 +58,7 @@ def test_error_paths_mirror_reference_driver():
         pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, 64, v_dtype=pkg.CFK_FP8_E4M3)  # not a reference mode
     with pytest.raises(pkg.CfkError):
         pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, 64, v_layout=1)
+    pkg.fmha_forward_plan(pkg.CFK_FP8_E4M3, 1, 1, 512, 512, 128, v_layout=1)
     # null params / null pointers
     lib = pkg.lib()
     assert lib.cfk_fmha_forward(None, None) == -1

@@ -153,12 +153,52 @@ def test_hybrid_exact_arithmetic():
         np.testing.assert_allclose(o.float().cpu().numpy(), ref, rtol=1.5e-3, atol=2e-4)
 
 
+@pytest.mark.parametrize("B,S,H,D", [(2, 512, 3, 128), (1, 384, 2, 64), (1, 256, 2, 256), (1, 4096, 2, 128)])
+def test_pretransposed_v_layout(B, S, H, D):
+    # V handed over as [B,D,H,S], the reference's offline transpose (fmha_forward.cu:514-532): same result as the
+    # [B,S,H,D] path up to the order of the fp32 accumulation
+    import torch
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    (qc, qs, qf), (kc, ks, kf), (vc, vs, vf) = (_quant(x) for x in (q, k, v))
+    vt = oracle.transpose_v_bdhs(vc)
+    assert vt.shape == (B, D, H, S)
+    o = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(vt), q_descale=qs, k_descale=ks, v_descale=vs,
+                         v_layout=pkg.fmha.CFK_V_BDHS)
+    o2 = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(vc), q_descale=qs, k_descale=ks, v_descale=vs)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    ref = oracle.attention_f32(qf, kf, vf)["O"]
+    err = max_abs(got, ref)
+    print(f"fp8 [B,D,H,S] V B={B} S={S} H={H} D={D}: max-abs {err:.3e}; vs [B,S,H,D] path {max_abs(got, o2.float().cpu().numpy()):.3e}")
+    assert err <= TOL_FP8
+    assert max_abs(got, o2.float().cpu().numpy()) <= 2e-3   # same P, same V, different summation order
+    if S >= 2048:
+        assert oracle.verify_tensor(got, ref, ERRPCT_FP8)[0]
+
+
+def test_pretransposed_v_exact_arithmetic():
+    rng = np.random.default_rng(13)
+    import torch
+    for D in (64, 128, 256):
+        B, S, H = 1, 384, 2
+        q = np.zeros((B, S, H, D), np.float32)
+        np.put_along_axis(q, rng.integers(0, D, (B, S, H, 4)), 1.0, axis=-1)
+        k = rng.integers(-1, 2, (B, S, H, D)).astype(np.float32)
+        v = rng.integers(-8, 9, (B, S, H, D)).astype(np.float32)
+        o = pkg.fmha_forward(to_dev(oracle.e4m3_encode(q)), to_dev(oracle.e4m3_encode(k)),
+                             to_dev(oracle.transpose_v_bdhs(oracle.e4m3_encode(v))), softmax_scale=float(np.log(2.0)),
+                             v_layout=pkg.fmha.CFK_V_BDHS)
+        torch.cuda.synchronize()
+        ref = oracle.attention_f32(q, k, v, alpha0=np.log(2.0))["O"]
+        np.testing.assert_allclose(o.float().cpu().numpy(), ref, rtol=1.5e-3, atol=2e-4)
+
+
 def test_unsupported_modes_report_errors():
     import torch
     x = torch.zeros((1, 128, 1, 64), dtype=torch.uint8, device="cuda:0")
-    xt = torch.zeros((1, 64, 1, 128), dtype=torch.uint8, device="cuda:0")
+    xt16 = torch.zeros((1, 64, 1, 128), dtype=torch.float16, device="cuda:0")
     with pytest.raises(pkg.CfkError) as e:
-        pkg.fmha_forward(x, x, xt, v_layout=pkg.fmha.CFK_V_BDHS)   # pre-transposed V is not built
+        pkg.fmha_forward(x, x, xt16, v_layout=pkg.fmha.CFK_V_BDHS)   # pre-transposed V is an e4m3-V layout
     assert e.value.code == -2
 
 
