@@ -52,9 +52,10 @@ int check_fmha(const cfk_fmha_fwd_params *p, cfk::FmhaPlan *plan, bool need_poin
   }
   const long long bh = (long long)p->batch * p->heads;
   if (bh > (1 << 24)) return fail(CFK_ERR_UNSUPPORTED, "batch*heads too large");
-  bool ok = p->dtype == CFK_FP16     ? cfk::plan_fmha_f16(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, plan)
-            : p->v_dtype == CFK_FP16 ? cfk::plan_fmha_hybrid(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, plan)
-                                     : cfk::plan_fmha_fp8(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, p->v_layout, plan);
+  const bool tap = p->dbg_s != nullptr;
+  bool ok = p->dtype == CFK_FP16     ? cfk::plan_fmha_f16(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, tap, plan)
+            : p->v_dtype == CFK_FP16 ? cfk::plan_fmha_hybrid(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, tap, plan)
+                                     : cfk::plan_fmha_fp8(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, p->v_layout, tap, plan);
   if (!ok) return fail(CFK_ERR_UNSUPPORTED, "no kernel for dtype %d head dim %d v_layout %d", p->dtype, p->head_dim, p->v_layout);
   // The kernels carry no masks, exactly like the reference (no bounds handling: fmha_forward.cu:361-372).
   if (p->seqlen_q % plan->block_m != 0)
@@ -114,6 +115,7 @@ int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
   a.k = p->k;
   a.v = p->v;
   a.o = p->o;
+  a.s_tap = p->dbg_s;
   a.row_max = p->dbg_row_max;
   a.row_sum = p->dbg_row_sum;
   a.B = p->batch;
@@ -122,6 +124,7 @@ int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
   a.Skv = p->seqlen_kv;
   a.v_layout = p->v_layout;
   hipError_t e;
+  a.s_scale = p->dtype == CFK_FP16 ? p->softmax_scale : p->softmax_scale * p->q_descale * p->k_descale;
   if (p->dtype == CFK_FP16) {
     a.scale_log2 = p->softmax_scale * kLog2e;
     a.out_scale = 1.0f;

@@ -13,10 +13,12 @@ struct FmhaArgs {
   const void *q, *k, *v;
   void *o;
   float *row_max;    // optional [B,H,Sq] tap: running max, log2 domain (reference: miOut)
+  float *s_tap;      // optional [B,H,Sq,Skv] tap: pre-softmax scores, natural domain     (reference: tensorS)
   float *row_sum;    // optional [B,H,Sq] tap: sum of exp2(t - max)     (reference: sPrimeOut)
   int32_t B, H, Sq, Skv;
   float scale_log2;  // softmax_scale * log2(e) * q_descale * k_descale
   float out_scale;   // v_descale (1 for fp16)
+  float s_scale;     // softmax_scale * q_descale * k_descale (scales the score tap)
   int32_t v_layout;  // 0 = [B,S,H,D], 1 = [B,D,H,S]
 };
 
@@ -25,12 +27,13 @@ struct FmhaPlan {
 };
 
 // Each launcher validates nothing: the C-ABI layer has already checked shapes against the plan.
+// `tap_s` (plan) / a.s_tap (launch) selects the build of the kernel that also writes the score tap.
 hipError_t launch_fmha_f16(const FmhaArgs &a, int head_dim, hipStream_t s);      // Q,K,V fp16
 hipError_t launch_fmha_fp8(const FmhaArgs &a, int head_dim, hipStream_t s);      // Q,K,V e4m3, P e4m3
 hipError_t launch_fmha_hybrid(const FmhaArgs &a, int head_dim, hipStream_t s);   // Q,K e4m3; P,V fp16
-bool plan_fmha_f16(int head_dim, int sq, int skv, int bh, FmhaPlan *p);
-bool plan_fmha_fp8(int head_dim, int sq, int skv, int bh, int v_layout, FmhaPlan *p);
-bool plan_fmha_hybrid(int head_dim, int sq, int skv, int bh, FmhaPlan *p);
+bool plan_fmha_f16(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *p);
+bool plan_fmha_fp8(int head_dim, int sq, int skv, int bh, int v_layout, bool tap_s, FmhaPlan *p);
+bool plan_fmha_hybrid(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *p);
 
 hipError_t launch_gemm_f16(int M, int N, int K, const void *A, const void *B, void *C, int layout, hipStream_t s);
 

@@ -59,17 +59,19 @@ namespace cfk {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef int int8v __attribute__((ext_vector_type(8)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int2v __attribute__((ext_vector_type(2)));
 
-template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_, bool VT_ = false>
+template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_, bool VT_ = false, bool TAP_S_ = false>
 struct FmhaCfg {
   static constexpr int D = D_, BN = BN_, NWAVES = NWAVES_;
   static constexpr int WPE = WPE_;                              // waves per SIMD the register budget is sized for
   static constexpr bool QK8 = QK8_, PV8 = PV8_;                 // e4m3 (true) or fp16 (false) operands of GEMM-I / II
   static constexpr bool VT = VT_;                               // V given pre-transposed, [B,D,H,S] (e4m3 only)
+  static constexpr bool TAP_S = TAP_S_;                         // also write the pre-softmax scores (debug build)
   static constexpr int T = NWAVES * 64;
   static constexpr int BM = NWAVES * 32;
   static constexpr int K_PITCH = D * (QK8 ? 1 : 2);             // bytes per LDS row, no padding
@@ -263,7 +265,20 @@ fmha_fwd_kernel(const FmhaArgs a) {
       }
   };
   // Row max of a finished S tile and the deferred rescale (online_softmax.h:123-165).  The branch is wave-uniform.
-  auto row_max_and_rescale = [&](const f32x16 (&sacc)[KB]) {
+  auto row_max_and_rescale = [&](const f32x16 (&sacc)[KB], int jt) {
+    if constexpr (C::TAP_S) {  // the reference's -DCOPYOUTMM0 dump (fmha_consumer.h:31-42), here already scaled
+      float *srow = a.s_tap + (((int64_t)b * a.H + h) * a.Sq + q0 + r) * (int64_t)a.Skv + (int64_t)jt * BN;
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key0 = C::VT ? 32 * g + 16 * kb + 4 * i : 32 * kb + 8 * i + 4 * g;  // a lane's 4 consecutive keys
+          f32x4 sv;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) sv[t] = sacc[kb][4 * i + t] * a.s_scale;
+          *(f32x4 *)(srow + key0) = sv;
+        }
+    }
     float mx = sacc[0][0];
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
@@ -353,7 +368,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
     if (HAS_NEXT) qk(P ^ 1, s_nxt);
     softmax_exp(s_cur, pb);
     pv(P, pb);
-    if (HAS_NEXT) row_max_and_rescale(s_nxt);
+    if (HAS_NEXT) row_max_and_rescale(s_nxt, j + 1);
     wait_lds_dma();   // this wave's copies have landed ...
     __syncthreads();  // ... and so have everybody else's; all reads of the stages about to be refilled are done
   };
@@ -366,7 +381,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
   wait_lds_dma();
   __syncthreads();
   qk(0, s_a);
-  row_max_and_rescale(s_a);
+  row_max_and_rescale(s_a, 0);
   __syncthreads();  // every wave is done with K stage 0 before step 0 overwrites it
 
   using std::integral_constant;

@@ -10,7 +10,8 @@
 //                            amax applies per-tensor amax/448 scales and passes the descales to the library
 //   --gemm2-fp8=true         with --prec-type=2: true = P and V in e4m3 too (the reference built with -DGEMM2FP8),
 //                            false = hybrid, Q,K e4m3 with fp16 P,V (the reference's default build, :446-450)
-//   --verify-all=false       also checks the row-max / row-sum taps (the reference's -DCOPYOUTMI build, :655-676)
+//   --verify-all=false       also checks the score / row-max / row-sum taps (the reference's -DCOPYOUTMM0
+//                            -DCOPYOUTMI build: gemm-check-1, max-check, sum-check, :640-676)
 //   --dump-dir=<dir>         writes q.bin k.bin v.bin o.bin (+ meta.txt) for an external checker
 //
 // The reference check follows the reference's: fp32 attention on the float up-casts of the (already quantised)
@@ -132,7 +133,7 @@ float e4m3_decode(uint8_t c) {
 // row max, then exp / row sum / P.V with the accumulator in registers.
 template <int D>
 __global__ void naive_attention(const float *Q, const float *K, const float *V, float *O, float *row_max, float *inv_sum,
-                                int B, int S, int H, float alpha) {
+                                float *scores, int B, int S, int H, float alpha) {
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (long long)B * H * S) return;
   const int m = (int)(idx % S);
@@ -151,6 +152,7 @@ __global__ void naive_attention(const float *Q, const float *K, const float *V, 
 #pragma unroll
     for (int d = 0; d < D; ++d) s += qr[d] * k0[n * ld + d];
     mx = fmaxf(mx, alpha * s);
+    if (scores) scores[idx * S + n] = alpha * s;
   }
   float acc[D];
 #pragma unroll
@@ -301,6 +303,11 @@ int main(int argc, char **argv) {
   HIP_CHECK(hipMalloc(&dout, n * 2));
   HIP_CHECK(hipMalloc(&dmi, (size_t)B * H * S * 4));
   HIP_CHECK(hipMalloc(&dsp, (size_t)B * H * S * 4));
+  // score tap (gemm-check-1): only with --verify-all and only when [B,H,S,S] fp32 stays under 2 GiB
+  const size_t n_scores = (size_t)B * H * S * S;
+  const bool check_scores = opt.ref_check && opt.verify_all && n_scores * 4 <= (2ull << 30);
+  float *dsc = nullptr;
+  if (check_scores) HIP_CHECK(hipMalloc(&dsc, n_scores * 4));
   HIP_CHECK(hipMemcpy(dq, qb.data(), n * esz, hipMemcpyHostToDevice));
   HIP_CHECK(hipMemcpy(dk, kb.data(), n * esz, hipMemcpyHostToDevice));
   HIP_CHECK(hipMemcpy(dv, vb.data(), n * vesz, hipMemcpyHostToDevice));
@@ -327,6 +334,7 @@ int main(int argc, char **argv) {
         p.k_descale = descale[1];
         p.v_descale = descale[2];
         if (taps) {
+          if (dsc) p.dbg_s = dsc + (size_t)i * Lb * H * S * S;
           p.dbg_row_max = dmi + (size_t)i * Lb * H * S;
           p.dbg_row_sum = dsp + (size_t)i * Lb * H * S;
         }
@@ -375,7 +383,8 @@ int main(int argc, char **argv) {
 
   int failed = 0;
   if (opt.ref_check) {
-    float *fq, *fk, *fv, *fo, *rmax, *rinv;
+    float *fq, *fk, *fv, *fo, *rmax, *rinv, *rsc = nullptr;
+    if (check_scores) HIP_CHECK(hipMalloc(&rsc, n_scores * 4));
     HIP_CHECK(hipMalloc(&fq, n * 4));
     HIP_CHECK(hipMalloc(&fk, n * 4));
     HIP_CHECK(hipMalloc(&fv, n * 4));
@@ -387,14 +396,24 @@ int main(int argc, char **argv) {
     HIP_CHECK(hipMemcpy(fv, hv.data(), n * 4, hipMemcpyHostToDevice));
     const long long rows = (long long)B * H * S;
     const dim3 grid((unsigned)((rows + 63) / 64)), block(64);
-    if (D == 64) hipLaunchKernelGGL(naive_attention<64>, grid, block, 0, 0, fq, fk, fv, fo, rmax, rinv, B, S, H, softmax_scale);
-    else if (D == 128) hipLaunchKernelGGL(naive_attention<128>, grid, block, 0, 0, fq, fk, fv, fo, rmax, rinv, B, S, H, softmax_scale);
-    else hipLaunchKernelGGL(naive_attention<256>, grid, block, 0, 0, fq, fk, fv, fo, rmax, rinv, B, S, H, softmax_scale);
+    if (D == 64) hipLaunchKernelGGL(naive_attention<64>, grid, block, 0, 0, fq, fk, fv, fo, rmax, rinv, rsc, B, S, H, softmax_scale);
+    else if (D == 128) hipLaunchKernelGGL(naive_attention<128>, grid, block, 0, 0, fq, fk, fv, fo, rmax, rinv, rsc, B, S, H, softmax_scale);
+    else hipLaunchKernelGGL(naive_attention<256>, grid, block, 0, 0, fq, fk, fv, fo, rmax, rinv, rsc, B, S, H, softmax_scale);
     HIP_CHECK(hipDeviceSynchronize());
     std::vector<float> ref(n), got(n);
     HIP_CHECK(hipMemcpy(ref.data(), fo, n * 4, hipMemcpyDeviceToHost));
     for (size_t i = 0; i < n; ++i) got[i] = (float)ho[i];
     const float err_expected = fp8 ? 0.001f : 0.0001f;  // :638-639
+    if (check_scores) {  // gemm-check-1 (:640-653); the library's tap is already scaled
+      std::vector<float> s_got(n_scores), s_ref(n_scores);
+      HIP_CHECK(hipMemcpy(s_got.data(), dsc, n_scores * 4, hipMemcpyDeviceToHost));
+      HIP_CHECK(hipMemcpy(s_ref.data(), rsc, n_scores * 4, hipMemcpyDeviceToHost));
+      const bool s_ok = verify_tensor(s_got, s_ref, opt.print_values, opt.print_diffs);
+      printf("gemm-check-1: %s\n", s_ok ? "Passed" : "Failed");
+      failed += !s_ok;
+    } else if (opt.verify_all) {
+      printf("gemm-check-1: skipped (score tensor above 2 GiB)\n");
+    }
     if (opt.verify_all) {
       const size_t nr = (size_t)rows;
       std::vector<float> mi(nr), sp(nr), rm(nr), ri(nr);
@@ -414,10 +433,10 @@ int main(int argc, char **argv) {
     const bool ok = verify_tensor(got, ref, opt.print_values, opt.print_diffs, err_expected);
     printf("gemm-check-2: %s\n", ok ? "Passed" : "Failed");
     failed += !ok;
-    hipFree(fq); hipFree(fk); hipFree(fv); hipFree(fo); hipFree(rmax); hipFree(rinv);
+    hipFree(fq); hipFree(fk); hipFree(fv); hipFree(fo); hipFree(rmax); hipFree(rinv); hipFree(rsc);
   }
   for (auto &s : streams)
     if (s) hipStreamDestroy(s);
-  hipFree(dq); hipFree(dk); hipFree(dv); hipFree(dout); hipFree(dmi); hipFree(dsp);
+  hipFree(dq); hipFree(dk); hipFree(dv); hipFree(dout); hipFree(dmi); hipFree(dsp); hipFree(dsc);
   return failed ? 3 : 0;
 }

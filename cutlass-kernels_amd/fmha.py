@@ -39,7 +39,7 @@ class FmhaFwdParams(ctypes.Structure):
         ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p), ("o", ctypes.c_void_p),
         ("softmax_scale", ctypes.c_float),
         ("q_descale", ctypes.c_float), ("k_descale", ctypes.c_float), ("v_descale", ctypes.c_float),
-        ("dbg_row_max", ctypes.c_void_p), ("dbg_row_sum", ctypes.c_void_p),
+        ("dbg_s", ctypes.c_void_p), ("dbg_row_max", ctypes.c_void_p), ("dbg_row_sum", ctypes.c_void_p),
     ]
 
 
@@ -92,7 +92,7 @@ def _check(rc):
 
 def make_params(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, q=0, k=0, v=0, o=0, softmax_scale=None,
                 q_descale=1.0, k_descale=1.0, v_descale=1.0, v_layout=CFK_V_BSHD, v_dtype=None,
-                dbg_row_max=0, dbg_row_sum=0) -> FmhaFwdParams:
+                dbg_row_max=0, dbg_row_sum=0, dbg_s=0) -> FmhaFwdParams:
     p = FmhaFwdParams()
     p.dtype = dtype
     p.v_dtype = dtype if v_dtype is None else v_dtype
@@ -101,6 +101,7 @@ def make_params(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, q=0, k=0, v=
     p.q, p.k, p.v, p.o = q or None, k or None, v or None, o or None
     p.softmax_scale = (1.0 / math.sqrt(head_dim)) if softmax_scale is None else softmax_scale
     p.q_descale, p.k_descale, p.v_descale = q_descale, k_descale, v_descale
+    p.dbg_s = dbg_s or None
     p.dbg_row_max = dbg_row_max or None
     p.dbg_row_sum = dbg_row_sum or None
     return p
@@ -122,12 +123,12 @@ def _stream_ptr(stream):
 
 
 def fmha_forward(q, k, v, o=None, softmax_scale=None, q_descale=1.0, k_descale=1.0, v_descale=1.0,
-                 v_layout=CFK_V_BSHD, row_max=None, row_sum=None, stream=None):
+                 v_layout=CFK_V_BSHD, row_max=None, row_sum=None, scores=None, stream=None):
     """O = softmax(scale * Q K^T) V on device tensors in [B,S,H,D] (D contiguous).
 
     q,k,v: torch CUDA tensors, float16, or float8_e4m3fn / uint8 holding e4m3 codes (v may be float16 with e4m3
     q,k: hybrid mode).  ``v`` is [B,D,H,S] when
-    ``v_layout == CFK_V_BDHS``.  Returns ``o`` (float16 [B,Sq,H,D]); launches asynchronously on ``stream``
+    ``v_layout == CFK_V_BDHS``.  ``row_max`` / ``row_sum`` / ``scores`` are the optional debug taps.  Returns ``o`` (float16 [B,Sq,H,D]); launches asynchronously on ``stream``
     (default: torch's current stream)."""
     import torch
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
@@ -162,10 +163,14 @@ def fmha_forward(q, k, v, o=None, softmax_scale=None, q_descale=1.0, k_descale=1
     for t in (row_max, row_sum):
         if t is not None and (t.dtype != torch.float32 or tuple(t.shape) != (B, H, Sq) or not t.is_contiguous()):
             raise ValueError("row_max/row_sum must be contiguous float32 [B,H,Sq]")
+    if scores is not None and (scores.dtype != torch.float32 or tuple(scores.shape) != (B, H, Sq, Skv)
+                               or not scores.is_contiguous()):
+        raise ValueError("scores must be contiguous float32 [B,H,Sq,Skv]")
     p = make_params(dtype, B, H, Sq, Skv, D, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), softmax_scale,
                     q_descale, k_descale, v_descale, v_layout, v_dtype=v_dtype,
                     dbg_row_max=row_max.data_ptr() if row_max is not None else 0,
-                    dbg_row_sum=row_sum.data_ptr() if row_sum is not None else 0)
+                    dbg_row_sum=row_sum.data_ptr() if row_sum is not None else 0,
+                    dbg_s=scores.data_ptr() if scores is not None else 0)
     _check(lib().cfk_fmha_forward(ctypes.byref(p), _stream_ptr(stream)))
     return o
 

@@ -68,6 +68,10 @@ typedef struct cfk_fmha_fwd_params {
   float q_descale;   /* fp8 per-tensor scales: real value = code value * descale.  1.0f reproduces the        */
   float k_descale;   /* reference, which applies no scaling (fmha_forward.cu:498-500).  Ignored for fp16.     */
   float v_descale;   /* ignored when v_dtype is CFK_FP16                                                      */
+  float *dbg_s;       /* optional tap, [B, H, S_q, S_kv] fp32: pre-softmax scores softmax_scale * Q K^T (natural
+                         domain, fp8 descales applied) -- the reference's tensorS under COPYOUTMM0
+                         (fmha_consumer.h:31-42), which it scales on the host before gemm-check-1
+                         (fmha_forward.cu:640-653).  Selects a debug build of the kernel (128-row tile); NULL = off */
   float *dbg_row_max; /* optional tap, [B, H, S_q] fp32: running row max in the log2 domain (score*scale*log2e),
                          the reference's miOut under COPYOUTMI (fmha_epilogue.h:7-46); NULL = off              */
   float *dbg_row_sum; /* optional tap, [B, H, S_q] fp32: row sum of exp2(t - max), not its reciprocal, the

@@ -24,10 +24,10 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_params_struct_matches_header_layout():
-    # 8 int32, 4 pointers, 4 floats, 2 pointers on LP64
-    assert ctypes.sizeof(pkg.fmha.FmhaFwdParams) == 8 * 4 + 4 * 8 + 4 * 4 + 2 * 8
+    # 8 int32, 4 pointers, 4 floats, 3 pointers on LP64
+    assert ctypes.sizeof(pkg.fmha.FmhaFwdParams) == 8 * 4 + 4 * 8 + 4 * 4 + 3 * 8
     assert pkg.fmha.FmhaFwdParams.q.offset == 32 and pkg.fmha.FmhaFwdParams.softmax_scale.offset == 64
-    assert pkg.fmha.FmhaFwdParams.dbg_row_max.offset == 80
+    assert pkg.fmha.FmhaFwdParams.dbg_s.offset == 80 and pkg.fmha.FmhaFwdParams.dbg_row_max.offset == 88
 
 
 def test_version_and_plan_without_gpu():

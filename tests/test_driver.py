@@ -74,6 +74,7 @@ def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
                f"--dump-dir={tmp_path}", *extra).stdout
     assert "CUTE_FMHA:" in out and "Gflop/s" in out
     assert "gemm-check-2: Passed" in out and "max-check: Passed" in out and "sum-check: Passed" in out
+    assert "gemm-check-1: Passed" in out
     assert f"K = {head}" in out and "QBLK = " in out
     # independent check of the dumped tensors against the CPU oracle
     q, k, v, o, p = _load_dump(str(tmp_path))

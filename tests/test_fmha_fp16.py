@@ -87,6 +87,21 @@ def test_row_max_and_row_sum_taps():
     np.testing.assert_allclose(1.0 / rs.cpu().numpy(), r["inv_sum"], rtol=1e-4)
 
 
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_score_tap(D):
+    # the reference's gemm-check-1 (fmha_forward.cu:640-653): pre-softmax scores against the oracle's, exact
+    # products of fp16 values accumulated in fp32
+    import torch
+    B, S, H = 2, 256, 2
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    sc = torch.full((B, H, S, S), -1.0, dtype=torch.float32, device="cuda:0")
+    got, (qf, kf, vf) = _run(q, k, v, scores=sc)
+    r = oracle.attention_f32(qf, kf, vf, want_scores=True)
+    assert max_abs(got, r["O"]) <= TOL_FP16
+    assert oracle.verify_tensor(sc.cpu().numpy(), r["S"])[0]
+    np.testing.assert_allclose(sc.cpu().numpy(), r["S"], rtol=1e-4, atol=1e-4)
+
+
 def test_kernel_matches_tiled_emulation_closely():
     # against the numpy emulation of the kernel-side algorithm (P rounded to fp16 per tile) the difference is
     # rounding noise of the fp16 output only

@@ -193,6 +193,29 @@ def test_pretransposed_v_exact_arithmetic():
         np.testing.assert_allclose(o.float().cpu().numpy(), ref, rtol=1.5e-3, atol=2e-4)
 
 
+@pytest.mark.parametrize("mode", ["fp8", "fp8_bdhs", "hybrid"])
+def test_score_tap(mode):
+    import torch
+    B, S, H, D = 1, 256, 2, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    (qc, qs, qf), (kc, ks, kf), (vc, vs, vf) = (_quant(x) for x in (q, k, v))
+    sc = torch.full((B, H, S, S), -1.0, dtype=torch.float32, device="cuda:0")
+    if mode == "hybrid":
+        vdev, kw, vf = to_dev(v.astype(np.float16)), {}, v.astype(np.float16).astype(np.float32)
+    elif mode == "fp8_bdhs":
+        vdev, kw = to_dev(oracle.transpose_v_bdhs(vc)), dict(v_descale=vs, v_layout=pkg.fmha.CFK_V_BDHS)
+    else:
+        vdev, kw = to_dev(vc), dict(v_descale=vs)
+    o = pkg.fmha_forward(to_dev(qc), to_dev(kc), vdev, q_descale=qs, k_descale=ks, scores=sc, **kw)
+    torch.cuda.synchronize()
+    r = oracle.attention_f32(qf, kf, vf, want_scores=True)
+    assert max_abs(o.float().cpu().numpy(), r["O"]) <= TOL_FP8
+    # the oracle multiplies the dequantised floats (each rounded after its descale), the kernel scales the exact
+    # product of the codes once: differences of a few 1e-4 on scores of magnitude ~1-5
+    assert oracle.verify_tensor(sc.cpu().numpy(), r["S"])[0]
+    np.testing.assert_allclose(sc.cpu().numpy(), r["S"], rtol=1e-3, atol=1e-3)
+
+
 def test_unsupported_modes_report_errors():
     import torch
     x = torch.zeros((1, 128, 1, 64), dtype=torch.uint8, device="cuda:0")
