@@ -81,3 +81,19 @@ def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
     ref = oracle.attention_f32(q, k, v)["O"]
     assert max_abs(o, ref) <= (TOL_FP16 if p == 1 else TOL_FP8)
     assert oracle.verify_tensor(o, ref, ERRPCT_FP16 if p == 1 else ERRPCT_FP8)[0]
+
+
+GEMM_DRIVER = os.path.join(ROOT, "cutlass-kernels_amd", "driver", "gemm")
+
+
+def test_gemm_driver_rejects_other_types():
+    r = subprocess.run([GEMM_DRIVER, "1"], capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "invalid type value" in r.stdout
+
+
+@pytest.mark.gpu
+def test_gemm_driver_runs_and_checks():
+    r = subprocess.run([GEMM_DRIVER, "3", "1024", "768", "512", "2", "check"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "CUTE_GEMM:" in r.stdout and "GFlop/s" in r.stdout and "L = 2" in r.stdout
+    assert r.stdout.count("Passed") == 2 and "Failed" not in r.stdout
