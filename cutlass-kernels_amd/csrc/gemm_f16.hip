@@ -115,41 +115,65 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
       for (int v = 0; v < 16; ++v) acc[mb][nb][v] = 0.f;
 
   const int k_tiles = K / BK;
+  // operand fetch for K-step s of the tile in LDS stage `st`
+  auto fetch = [&](const char *st, int s, half8 (&aop)[4], half8 (&bop)[2]) {
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      if (!NN) {
+        bop[nb] = *(const half8 *)(st + b_rd[s] + nb * 32 * 128);
+      } else {
+        union {
+          struct { short4v lo, hi; } p;
+          half8 h;
+        } u;
+        const char *bp = st + bt_rd[nb] + s * 16 * 512;
+        u.p.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp));
+        u.p.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp + 4 * 512));
+        bop[nb] = u.h;
+      }
+    }
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) aop[mb] = *(const half8 *)(st + a_rd[s] + mb * 32 * 128);
+  };
+  auto mma = [&](const half8 (&aop)[4], const half8 (&bop)[2]) {
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)  // transposed block: MFMA rows = n (B operand first), columns = m
+        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop[mb], acc[mb][nb], 0, 0, 0);
+  };
+
   load_stage(0, 0);
   wait_lds_dma();
   __syncthreads();
+  half8 a0[4], b0[2], a1[4], b1[2];  // two operand register sets: K-step s+1 is fetched while K-step s multiplies
+  fetch(smem, 0, a0, b0);
   for (int kt = 0; kt < k_tiles; ++kt) {
     const int stage = kt & 1;
     load_stage(kt + 1 < k_tiles ? kt + 1 : kt, stage ^ 1);
     const char *st = smem + stage * STAGE;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      half8 bop[2];
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
-        if (!NN) {
-          bop[nb] = *(const half8 *)(st + b_rd[s] + nb * 32 * 128);
-        } else {
-          union {
-            struct { short4v lo, hi; } p;
-            half8 h;
-          } u;
-          const char *bp = st + bt_rd[nb] + s * 16 * 512;
-          u.p.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp));
-          u.p.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp + 4 * 512));
-          bop[nb] = u.h;
-        }
-      }
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb) {
-        const half8 aop = *(const half8 *)(st + a_rd[s] + mb * 32 * 128);
-#pragma unroll
-        for (int nb = 0; nb < 2; ++nb)  // transposed block: MFMA rows = n (B operand first), columns = m
-          acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop, acc[mb][nb], 0, 0, 0);
-      }
-    }
+    // sched_barrier(0): the compiler's scheduler would otherwise sink each fetch down to its first use and expose
+    // the LDS latency in front of every multiply
+    fetch(st, 1, a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(a0, b0);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(st, 2, a0, b0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(st, 3, a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(a0, b0);
+    __builtin_amdgcn_sched_barrier(0);
     wait_lds_dma();
-    __syncthreads();
+    __syncthreads();  // next stage has landed for everybody; this stage may be refilled after the last reads below
+    // first K-step of the next tile is fetched before the last multiply of this one (the barrier above already
+    // guarantees the data; the refill of THIS stage only starts after the next barrier)
+    fetch(smem + (stage ^ 1) * STAGE, 0, a0, b0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma(a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // ---- epilogue: lane (m = r, g) holds n = 8i + 4g + j of each block
