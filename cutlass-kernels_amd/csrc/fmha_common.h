@@ -57,6 +57,10 @@ __device__ __forceinline__ int xcd_remap(int wg, int n) {
 __device__ __forceinline__ void lds_dma16(const void *gptr, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr) : "memory");
 }
+// The same copy addressed as wave-uniform base (SGPR pair) + per-lane 32-bit byte offset: no 64-bit vector add per copy.
+__device__ __forceinline__ void lds_dma16(const void *base, uint32_t lane_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(base) : "memory");
+}
 __device__ __forceinline__ void wait_lds_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 }  // namespace cfk

@@ -180,13 +180,13 @@ fmha_fwd_kernel(const FmhaArgs a) {
     const char *gt = Kp + (size_t)jt * ((size_t)BN * k_ld);
 #pragma unroll
     for (int i = 0; i < C::K_IPW; ++i)
-      lds_dma16(gt + goff_k[i], lds_base + C::K_ST0 + stage * C::K_TILE + (i * C::NWAVES + wave) * 1024);
+      lds_dma16(gt, goff_k[i], lds_base + C::K_ST0 + stage * C::K_TILE + (i * C::NWAVES + wave) * 1024);
   };
   auto load_v = [&](int jt, int stage) {
     const char *gt = C::VT ? Vp + (size_t)jt * BN : Vp + (size_t)jt * ((size_t)BN * v_ld);
 #pragma unroll
     for (int i = 0; i < C::V_IPW; ++i)
-      lds_dma16(gt + goff_v[i], lds_base + C::V_ST0 + stage * C::V_TILE + (i * C::NWAVES + wave) * 1024);
+      lds_dma16(gt, goff_v[i], lds_base + C::V_ST0 + stage * C::V_TILE + (i * C::NWAVES + wave) * 1024);
   };
 
   // ---- Q: B operand of S^T, resident in VGPRs.  fp16: lane (r, g), K-step s holds Q[q0+r][16s + 8g .. +8);
@@ -241,6 +241,20 @@ fmha_fwd_kernel(const FmhaArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
   float m_ref = -INFINITY, m_true = -INFINITY, l_run = 0.f;  // softmax reference point, true running max, running sum
+  // e4m3 P: the row sum is taken on the MFMA pipe, which has cycles to spare there while the VALU does not.  One
+  // 16x16x128 MFMA per 64 keys multiplies P^T (the same registers that feed the second GEMM) by a 0/1 matrix:
+  // B lane (n = lane%16, block lane/16) is this kernel's lane (q = lane%32, g = lane/32), i.e. the 32 keys of query
+  // n + 16*(block%2); A[m][block] = 1 iff block%2 == (m/4)%2, so output rows 4i..4i+3 of lane (n, i = lane/16) all
+  // hold the sum over BOTH key halves of query n + 16*(i%2) = lane%32: every lane ends up with the sum of its own
+  // query, no exchange needed.  It sums P as rounded to e4m3, the weights the second GEMM really applies.
+  constexpr bool MFMA_SUM = PV8 && D <= 128;  // head dim 256 has no registers to spare, and twice the MFMA work per key
+  f32x4 l_acc = {0.f, 0.f, 0.f, 0.f};
+  int8v sum_a;
+  {
+    const int one4 = (((lane >> 4) & 1) == ((lane >> 2) & 1)) ? 0x38383838 : 0;  // e4m3 1.0 = 0x38
+#pragma unroll
+    for (int t = 0; t < 8; ++t) sum_a[t] = one4;
+  }
 
   // S^T = K . Q^T for the K tile in LDS stage `stage`
   auto qk = [&](int stage, f32x16 (&sacc)[KB]) {
@@ -291,6 +305,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
       const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
       m_ref = m_new;
       l_run *= alpha;
+      if constexpr (MFMA_SUM) l_acc *= alpha;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -309,10 +324,12 @@ fmha_fwd_kernel(const FmhaArgs a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           p[t] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][4 * w + t], c_log2, -m_ref));
-          rs += p[t];
+          if constexpr (!MFMA_SUM) rs += p[t];
         }
         if constexpr (PV8) {  // slot 16 kb + 4 w + t
-          int packed = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], 0, false);
+          // the two converts overwrite both halves of the word: its old content is irrelevant, and handing in
+          // the bits of p[0] (dead after this instruction) lets the result take p[0]'s register without a move
+          int packed = __builtin_amdgcn_cvt_pk_fp8_f32(p[0], p[1], __builtin_bit_cast(int, p[0]), false);
           pb[kb / 2][(kb % 2) * 4 + w] = __builtin_amdgcn_cvt_pk_fp8_f32(p[2], p[3], packed, true);
         } else {              // K-step 2 kb + w / 2, slot 4 (w % 2) + t
 #pragma unroll
@@ -324,6 +341,11 @@ fmha_fwd_kernel(const FmhaArgs a) {
   // O^T += V^T . P^T for the V tile in LDS stage `stage`
   auto pv = [&](int stage, const PReg (&pb)[PS]) {
     const char *vt = smem + C::V_ST0 + stage * C::V_TILE;
+    if constexpr (MFMA_SUM) {
+#pragma unroll
+      for (int ps = 0; ps < PS; ++ps)
+        l_acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(sum_a, pb[ps], l_acc, 0, 0, 0, 0, 0, 0);
+    }
 #pragma unroll
     for (int ps = 0; ps < PS; ++ps)
 #pragma unroll
@@ -398,7 +420,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
   }
 
   // ---- epilogue: O = out_scale * O / l (online_softmax.h:59-85), fp16, [B,S,H,D]; a lane holds 4 consecutive d
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float l_tot = MFMA_SUM ? l_acc[0] : l_run + __shfl_xor(l_run, 32, 64);
   const float inv = a.out_scale / l_tot;
   const int qrow = q0 + r;
   _Float16 *orow = Op + (int64_t)qrow * ld;

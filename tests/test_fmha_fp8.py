@@ -100,10 +100,13 @@ def test_taps_and_invariants():
     r = oracle.attention_f32(qf, kf, vf, want_stats=True)
     # max-check / sum-check (fmha_forward.cu:655-676); scores are exact products of e4m3 values in fp32
     np.testing.assert_allclose(rm.cpu().numpy() / oracle.LOG2E, r["row_max"], rtol=1e-4, atol=1e-4)
-    np.testing.assert_allclose(1.0 / rs.cpu().numpy(), r["inv_sum"], rtol=1e-3)
-    # V = 1 -> O ~ 1 (P is rounded to e4m3 after the fp32 row sum)
+    # the e4m3 kernel sums the weights AS ROUNDED to e4m3 (the ones the second GEMM applies; the reference sums them
+    # in fp32 before the cast, online_softmax.h:173-206): rounding is unbiased, so the two sums agree to well under 1 %
+    np.testing.assert_allclose(1.0 / rs.cpu().numpy(), r["inv_sum"], rtol=1e-2)
+    # V = 1 -> O = 1 up to fp16 rounding: numerator and denominator add up the same rounded weights.  Also pins the
+    # lane mapping of the row-sum MFMA (sums landing on another query's lane would break this)
     ones, _ = _run(q, k, np.ones_like(v))
-    assert max_abs(ones, 1.0) <= 2e-2
+    assert max_abs(ones, 1.0) <= 1e-3
     # a common permutation of the keys (pins the V-tile layout transform: wrong key order in V would show here
     # and in every other test)
     perm = np.random.default_rng(5).permutation(S)
