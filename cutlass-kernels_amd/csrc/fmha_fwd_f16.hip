@@ -5,8 +5,9 @@ namespace cfk {
 namespace {
 
 // "small" = 4 waves x 32 query rows (two workgroups share a CU), "large" = 8 waves x 32 rows (one workgroup per CU,
-// half the K/V traffic per query row); both run two waves per SIMD.
-using Cfg64S = FmhaCfg<64, 64, 4, 2, false, false>;
+// half the K/V traffic per query row); both run two waves per SIMD, except head dim 64, whose small tile fits three
+// (154 registers) and is the faster one for it.
+using Cfg64S = FmhaCfg<64, 64, 4, 3, false, false>;
 using Cfg64L = FmhaCfg<64, 64, 8, 2, false, false>;
 using Cfg128S = FmhaCfg<128, 64, 4, 2, false, false>;
 using Cfg128L = FmhaCfg<128, 64, 8, 2, false, false>;
@@ -27,10 +28,9 @@ bool dispatch(int head_dim, int sq, int bh, bool tap_s, F &&f) {
       default: return false;
     }
   }
-  const bool large = use_large_tile(sq, bh);
   switch (head_dim) {
-    case 64: large ? f(Cfg64L{}) : f(Cfg64S{}); return true;
-    case 128: large ? f(Cfg128L{}) : f(Cfg128S{}); return true;
+    case 64: use_large_tile(sq, bh, false) ? f(Cfg64L{}) : f(Cfg64S{}); return true;
+    case 128: use_large_tile(sq, bh) ? f(Cfg128L{}) : f(Cfg128S{}); return true;
     case 256: f(Cfg256S{}); return true;
     default: return false;
   }

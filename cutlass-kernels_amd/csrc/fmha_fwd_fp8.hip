@@ -5,7 +5,7 @@
 namespace cfk {
 namespace {
 
-using Cfg64S = FmhaCfg<64, 64, 4, 2, true, true>;
+using Cfg64S = FmhaCfg<64, 64, 4, 3, true, true>;  // three waves per SIMD: the VALU-bound softmax gains from every extra wave
 using Cfg128S = FmhaCfg<128, 64, 4, 2, true, true>;
 using Cfg128L = FmhaCfg<128, 64, 8, 2, true, true>;
 using Cfg256S = FmhaCfg<256, 64, 4, 1, true, true>;  // O (128) + S (64) + Q (32) registers: one wave per SIMD

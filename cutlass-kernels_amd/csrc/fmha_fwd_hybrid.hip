@@ -6,7 +6,7 @@
 namespace cfk {
 namespace {
 
-using Cfg64S = FmhaCfg<64, 64, 4, 2, true, false>;
+using Cfg64S = FmhaCfg<64, 64, 4, 3, true, false>;
 using Cfg128S = FmhaCfg<128, 64, 4, 2, true, false>;
 using Cfg128L = FmhaCfg<128, 64, 8, 2, true, false>;
 using Cfg256S = FmhaCfg<256, 32, 4, 1, true, false>;
