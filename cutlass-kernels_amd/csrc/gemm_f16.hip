@@ -7,9 +7,14 @@
 // NN = B is K x N, N-contiguous (the literal C = A.B), whose B operand is read with ds_read_b64_tr_b16 exactly as V
 // is in the attention kernel.  The reference writes C column-major (:386-389); C is row-major here.
 //
-// Workgroup = 8 waves on a 256 x 256 macro tile, BK = 64, two LDS stages (A 32 KB + B 32 KB each).  Wave (wm, wn)
-// of a 2 x 4 grid owns 128 x 64 of C as 4 x 2 MFMA blocks.  The MFMA computes the TRANSPOSED block
-// (rows = n, columns = m) so that a lane ends up with 4 consecutive n of one row m: 8-byte row-major stores.
+// Workgroup = 4 waves (one per SIMD) on a 256 x 256 macro tile; wave (wm, wn) of a 2 x 2 grid owns 128 x 128 of C as
+// 4 x 4 MFMA blocks, its 256 accumulator registers in the AGPR half of the register file.  K tiles are 32 deep and go
+// through a ring of four LDS stages (32 KB each: A 16 KB + B 16 KB): the copy of tile kt+3 is issued, one 1 KB piece
+// after every four MFMAs, while tile kt multiplies.  Measured on MI355X, M=N=K=8192: the spread-out copies are worth
+// +15 % when the operands are constant (1.50 PFLOP/s; copies issued back to back fill the memory pipeline's queue and
+// stall the wave, and with one wave per SIMD the MFMA pipe with it); with U(-1,1) operands the board is power-limited
+// and every variant lands at 1.10-1.16 PFLOP/s.  The MFMA computes the TRANSPOSED block (rows = n, columns = m) so
+// that a lane ends up with 4 consecutive n of one row m: 8-byte row-major stores.
 #include <type_traits>
 
 #include "fmha_common.h"
@@ -22,20 +27,20 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 
-constexpr int BM = 256, BN = 256, BK = 64, NWAVES = 8, T = NWAVES * 64;
-constexpr int A_TILE = BM * BK * 2;            // 32 KB, rows of 128 B (K-contiguous)
-constexpr int B_TILE = BN * BK * 2;            // 32 KB: TN rows of 128 B (n rows); NN rows of 512 B (k rows)
-constexpr int STAGE = A_TILE + B_TILE;
-constexpr int LDS_BYTES = 2 * STAGE;
+constexpr int BM = 256, BN = 256;
 
-// 128-byte rows (two rows per 256-byte bank period): 16 consecutive rows at one 16-byte chunk index must spread
-// over all banks -> the 8 rows of equal parity get 8 distinct XOR values
-__device__ __forceinline__ int swz128(int row) { return (row >> 1) & 7; }
+// K-contiguous rows of PITCH bytes (128: two rows per 256-byte bank period; 64: four): 16 consecutive rows at one
+// 16-byte chunk index must spread over all banks -> rows at the same place in the period get distinct XOR values
+template <int PITCH>
+__device__ __forceinline__ int swz_k(int row) { return PITCH == 128 ? (row >> 1) & 7 : (row >> 2) & 3; }
 // 512-byte rows read with ds_read_b64_tr_b16 (4 consecutive k x 64 contiguous bytes)
 __device__ __forceinline__ int swz512(int row) { return (row & 3) << 2; }
 
-template <bool NN>
-__global__ void __launch_bounds__(T) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// WN = waves along n (2 along m always): 2 -> 4 waves of 128 x 128, one per SIMD (the shipped shape; a third less
+// LDS traffic per MFMA than 4 -> 8 waves of 128 x 64, two per SIMD).
+// BK = depth of a K tile, NS = LDS stages (copies run NS-1 tiles ahead of the multiply).
+template <bool NN, int WN, int BK, int NS>
+__global__ void __launch_bounds__(2 * WN * 64) __attribute__((amdgpu_waves_per_eu(WN / 2, WN / 2)))
 gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, _Float16 *__restrict__ C, int M, int N,
                 int K) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -43,7 +48,15 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, g = lane >> 5;
-  const int wm = wave >> 2, wn = wave & 3;
+  constexpr int NWAVES = 2 * WN;
+  constexpr int NB = BN / WN / 32;     // 32-column blocks per wave
+  constexpr int PITCH = BK * 2;        // bytes per K-contiguous LDS row
+  constexpr int A_TILE = BM * PITCH;   // TN: B tile likewise (n rows); NN: BK rows (k) of 512 B
+  constexpr int STAGE = 2 * A_TILE;
+  constexpr int CPW = A_TILE / 1024 / NWAVES;  // 1 KB copies per wave and operand tile
+  constexpr int RPC = 1024 / PITCH;    // rows per copy
+  constexpr int KS = BK / 16;          // 16-deep K-steps per tile
+  const int wm = wave / WN, wn = wave % WN;
 
   // tile order: groups of 8 tile rows, column-major inside a group, so concurrently running workgroups share A and
   // B panels in L2; workgroup ids are first remapped so that each XCD owns a contiguous range of that order
@@ -65,12 +78,12 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
 
   // ---- global -> LDS copies, 16 B per lane, 1 KB per wave-wide copy
   // A (and B in TN): 8 rows of 128 B per copy; 32 copies per tile, 4 per wave.
-  uint32_t goff_a[4], goff_b[4];
+  uint32_t goff_a[CPW], goff_b[CPW];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = (i * NWAVES + wave) * 8 + (lane >> 3);
-    const int cp = lane & 7;
-    goff_a[i] = (uint32_t)row * (uint32_t)(K * 2) + (uint32_t)((cp ^ swz128(row)) * 16);
+  for (int i = 0; i < CPW; ++i) {
+    const int row = (i * NWAVES + wave) * RPC + lane / (PITCH / 16);
+    const int cp = lane % (PITCH / 16);
+    goff_a[i] = (uint32_t)row * (uint32_t)(K * 2) + (uint32_t)((cp ^ swz_k<PITCH>(row)) * 16);
     if (!NN) {
       goff_b[i] = goff_a[i];
     } else {  // B tile is BK rows (k) of 512 B (256 n): 2 rows per copy
@@ -83,44 +96,44 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
     const char *ga = Ap + (size_t)kt * (BK * 2);
     const char *gb = NN ? Bp + (size_t)kt * BK * (size_t)(N * 2) : Bp + (size_t)kt * (BK * 2);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_dma16(ga + goff_a[i], lds_base + stage * STAGE + (i * NWAVES + wave) * 1024);
+    for (int i = 0; i < CPW; ++i) lds_dma16(ga + goff_a[i], lds_base + stage * STAGE + (i * NWAVES + wave) * 1024);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_dma16(gb + goff_b[i], lds_base + stage * STAGE + A_TILE + (i * NWAVES + wave) * 1024);
+    for (int i = 0; i < CPW; ++i) lds_dma16(gb + goff_b[i], lds_base + stage * STAGE + A_TILE + (i * NWAVES + wave) * 1024);
   };
 
   // ---- LDS read addresses.  K-step s (16 deep): lane (r, g) needs k = 16s + 8g .. +8 of its row.
-  int a_rd[4], b_rd[4];
+  int a_rd[KS], b_rd[KS];
 #pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    a_rd[s] = (wm * 128 + r) * 128 + (((2 * s + g) ^ swz128(r)) * 16);          // + 32*128 per m block
-    b_rd[s] = A_TILE + (wn * 64 + r) * 128 + (((2 * s + g) ^ swz128(r)) * 16);  // + 32*128 per n block (TN)
+  for (int s = 0; s < KS; ++s) {
+    a_rd[s] = (wm * 128 + r) * PITCH + (((2 * s + g) ^ swz_k<PITCH>(r)) * 16);               // + 32 rows per m block
+    b_rd[s] = A_TILE + (wn * NB * 32 + r) * PITCH + (((2 * s + g) ^ swz_k<PITCH>(r)) * 16);  // + 32 rows per n block (TN)
   }
   // NN: B^T operand via ds_read_b64_tr_b16 from [k][n] rows (see the V operand of the attention kernel)
   const int li = lane & 15;
   const int bk_row = 8 * g + (li >> 2);                                // + 16 s + 4 h2: slot t of lane g is k = 16s + 8g + t, as in A
-  const int bn_col = wn * 64 + 16 * ((lane >> 4) & 1) + 4 * (li & 3);  // + 32 nb
-  int bt_rd[2];
+  const int bn_col = wn * NB * 32 + 16 * ((lane >> 4) & 1) + 4 * (li & 3);  // + 32 nb
+  int bt_rd[NB];
 #pragma unroll
-  for (int nb = 0; nb < 2; ++nb) {
+  for (int nb = 0; nb < NB; ++nb) {
     const int c = (bn_col + 32 * nb) >> 3;
     bt_rd[nb] = A_TILE + bk_row * 512 + ((c ^ swz512(bk_row)) * 16) + (bn_col & 7) * 2;
   }
 
-  f32x16 acc[4][2];
+  f32x16 acc[4][NB];
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[mb][nb][v] = 0.f;
 
   const int k_tiles = K / BK;
   // operand fetch for K-step s of the tile in LDS stage `st`
-  auto fetch = [&](const char *st, int s, half8 (&aop)[4], half8 (&bop)[2]) {
+  auto fetch = [&](const char *st, int s, half8 (&aop)[4], half8 (&bop)[NB]) {
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int nb = 0; nb < NB; ++nb) {
       if (!NN) {
-        bop[nb] = *(const half8 *)(st + b_rd[s] + nb * 32 * 128);
+        bop[nb] = *(const half8 *)(st + b_rd[s] + nb * 32 * PITCH);
       } else {
         union {
           struct { short4v lo, hi; } p;
@@ -133,55 +146,76 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
       }
     }
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) aop[mb] = *(const half8 *)(st + a_rd[s] + mb * 32 * 128);
+    for (int mb = 0; mb < 4; ++mb) aop[mb] = *(const half8 *)(st + a_rd[s] + mb * 32 * PITCH);
   };
-  auto mma = [&](const half8 (&aop)[4], const half8 (&bop)[2]) {
+  // One copy (index c of the 2*CPW a wave issues per tile: first the A ones, then the B ones) of the tile at
+  // ga / gb into stage `fill`
+  auto load_copy = [&](const char *ga, const char *gb, int fill, int c) {
+    if (c < CPW) lds_dma16(ga + goff_a[c], lds_base + fill * STAGE + (c * NWAVES + wave) * 1024);
+    else lds_dma16(gb + goff_b[c - CPW], lds_base + fill * STAGE + A_TILE + ((c - CPW) * NWAVES + wave) * 1024);
+  };
+  // The multiplies of one K-step, with the copies [c0, c1) of the tile being prefetched spread between them: the
+  // L1 takes a 1 KB copy apart into sixteen 64-byte accesses, so copies issued back to back fill the memory
+  // pipeline's queue and stall the wave (and with it the MFMA pipe) at the next one.
+  auto mma = [&](const half8 (&aop)[4], const half8 (&bop)[NB], const char *ga, const char *gb, int fill, int c0, int c1) {
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+    for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb)  // transposed block: MFMA rows = n (B operand first), columns = m
+      for (int nb = 0; nb < NB; ++nb)  // transposed block: MFMA rows = n (B operand first), columns = m
         acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop[mb], acc[mb][nb], 0, 0, 0);
+#pragma unroll
+      for (int c = c0 + mb; c < c1; c += 4) load_copy(ga, gb, fill, c);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
-  load_stage(0, 0);
+  // Copies per wave and tile, and how they spread over the K-steps of the tile that is multiplied meanwhile.  With
+  // two stages the tile being copied is needed right after this tile's barrier, so its copies go with the first KS-1
+  // steps; with more stages they go with all KS steps and the wait leaves the younger tiles in flight.
+  constexpr int CPT = 2 * CPW;
+  constexpr int PER_STEP = NS == 2 ? (CPT + KS - 2) / (KS - 1) : CPT / KS;
+  constexpr int IN_FLIGHT = NS == 2 ? 0 : (NS - 3) * CPT + (KS - 1) * PER_STEP;
+  auto wait_tile = [&]() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT) : "memory"); };
+#pragma unroll
+  for (int t0 = 0; t0 < NS - 1; ++t0) load_stage(t0 < k_tiles ? t0 : k_tiles - 1, t0);
   wait_lds_dma();
   __syncthreads();
-  half8 a0[4], b0[2], a1[4], b1[2];  // two operand register sets: K-step s+1 is fetched while K-step s multiplies
-  fetch(smem, 0, a0, b0);
+  half8 aop[2][4], bop[2][NB];  // two operand register sets: K-step s+1 is fetched while K-step s multiplies
+  fetch(smem, 0, aop[0], bop[0]);
+  int stage = 0;
   for (int kt = 0; kt < k_tiles; ++kt) {
-    const int stage = kt & 1;
-    load_stage(kt + 1 < k_tiles ? kt + 1 : kt, stage ^ 1);
+    // the stage the previous tile was read from (its last reads were issued before that tile's barrier) is refilled
+    // with tile kt+NS-1 (clamped at the end: a surplus copy rewrites a stage nobody reads any more)
+    const int fill = stage == 0 ? NS - 1 : stage - 1;
+    const int ld_t = kt + NS - 1 < k_tiles ? kt + NS - 1 : k_tiles - 1;
+    const char *ga = Ap + (size_t)ld_t * (BK * 2);
+    const char *gb = NN ? Bp + (size_t)ld_t * BK * (size_t)(N * 2) : Bp + (size_t)ld_t * (BK * 2);
     const char *st = smem + stage * STAGE;
+    const int nstage = stage + 1 == NS ? 0 : stage + 1;
     // sched_barrier(0): the compiler's scheduler would otherwise sink each fetch down to its first use and expose
     // the LDS latency in front of every multiply
-    fetch(st, 1, a1, b1);
+#pragma unroll
+    for (int s2 = 0; s2 + 1 < KS; ++s2) {
+      fetch(st, s2 + 1, aop[(s2 + 1) & 1], bop[(s2 + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+      mma(aop[s2 & 1], bop[s2 & 1], ga, gb, fill, s2 * PER_STEP, (s2 + 1) * PER_STEP < CPT ? (s2 + 1) * PER_STEP : CPT);
+    }
+    wait_tile();
+    __syncthreads();  // the next tile has landed for everybody
+    // first K-step of the next tile is fetched before the last multiply of this one
+    fetch(smem + nstage * STAGE, 0, aop[0], bop[0]);
     __builtin_amdgcn_sched_barrier(0);
-    mma(a0, b0);
-    __builtin_amdgcn_sched_barrier(0);
-    fetch(st, 2, a0, b0);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(a1, b1);
-    __builtin_amdgcn_sched_barrier(0);
-    fetch(st, 3, a1, b1);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(a0, b0);
-    __builtin_amdgcn_sched_barrier(0);
-    wait_lds_dma();
-    __syncthreads();  // next stage has landed for everybody; this stage may be refilled after the last reads below
-    // first K-step of the next tile is fetched before the last multiply of this one (the barrier above already
-    // guarantees the data; the refill of THIS stage only starts after the next barrier)
-    fetch(smem + (stage ^ 1) * STAGE, 0, a0, b0);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(a1, b1);
-    __builtin_amdgcn_sched_barrier(0);
+    mma(aop[(KS - 1) & 1], bop[(KS - 1) & 1], ga, gb, fill, NS == 2 ? CPT : (KS - 1) * PER_STEP, CPT);
+    stage = nstage;
   }
+  wait_lds_dma();  // no copy may still be writing LDS when the workgroup retires
 
   // ---- epilogue: lane (m = r, g) holds n = 8i + 4g + j of each block
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
-    _Float16 *crow = C + (int64_t)(m0 + wm * 128 + mb * 32 + r) * N + n0 + wn * 64;
+    _Float16 *crow = C + (int64_t)(m0 + wm * 128 + mb * 32 + r) * N + n0 + wn * NB * 32;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         half4 o4;
@@ -192,16 +226,17 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
   }
 }
 
-template <bool NN>
+template <bool NN, int WN, int BK, int NS>
 hipError_t launch(int M, int N, int K, const void *A, const void *B, void *C, hipStream_t s) {
   static bool attr_done = false;
-  auto kern = gemm_f16_kernel<NN>;
+  auto kern = gemm_f16_kernel<NN, WN, BK, NS>;
+  constexpr int LDS_BYTES = NS * 2 * BM * BK * 2;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  hipLaunchKernelGGL(kern, dim3((M / BM) * (N / BN)), dim3(T), LDS_BYTES, s, (const _Float16 *)A, (const _Float16 *)B,
+  hipLaunchKernelGGL(kern, dim3((M / BM) * (N / BN)), dim3(2 * WN * 64), LDS_BYTES, s, (const _Float16 *)A, (const _Float16 *)B,
                      (_Float16 *)C, M, N, K);
   return hipGetLastError();
 }
@@ -209,7 +244,7 @@ hipError_t launch(int M, int N, int K, const void *A, const void *B, void *C, hi
 }  // namespace
 
 hipError_t launch_gemm_f16(int M, int N, int K, const void *A, const void *B, void *C, int layout, hipStream_t s) {
-  return layout == 0 ? launch<false>(M, N, K, A, B, C, s) : launch<true>(M, N, K, A, B, C, s);
+  return layout == 0 ? launch<false, 2, 32, 4>(M, N, K, A, B, C, s) : launch<true, 2, 32, 4>(M, N, K, A, B, C, s);
 }
 
 }  // namespace cfk
