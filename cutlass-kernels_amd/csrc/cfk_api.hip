@@ -142,18 +142,57 @@ int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
   return CFK_OK;
 }
 
-int cfk_gemm_f16(int32_t M, int32_t N, int32_t K, const void *A, const void *B, void *C, int32_t layout, void *stream) {
-  if (M <= 0 || N <= 0 || K <= 0) return fail(CFK_ERR_INVALID_ARG, "M, N, K must be positive (got %d, %d, %d)", M, N, K);
-  if (!A || !B || !C) return fail(CFK_ERR_INVALID_ARG, "A, B, C must be non-NULL device pointers");
-  if (layout != CFK_GEMM_TN && layout != CFK_GEMM_NN) return fail(CFK_ERR_INVALID_ARG, "unknown GEMM layout %d", layout);
-  if (M % 256 || N % 256 || K % 64)
-    return fail(CFK_ERR_UNSUPPORTED, "M and N must be multiples of 256 and K of 64 (got %d, %d, %d)", M, N, K);
+int cfk_gemm(const cfk_gemm_params *p, void *stream) {
+  if (!p) return fail(CFK_ERR_INVALID_ARG, "params is NULL");
+  if (p->dtype != CFK_FP16 && p->dtype != CFK_FP32)
+    return fail(CFK_ERR_INVALID_ARG, "GEMM dtype must be CFK_FP16 or CFK_FP32 (got %d)", p->dtype);
+  if (p->m <= 0 || p->n <= 0 || p->k <= 0 || p->batch <= 0)
+    return fail(CFK_ERR_INVALID_ARG, "M, N, K, batch must be positive (got %d, %d, %d, %d)", p->m, p->n, p->k, p->batch);
+  if (!p->a || !p->b || !p->d) return fail(CFK_ERR_INVALID_ARG, "A, B, D must be non-NULL device pointers");
+  if (p->layout != CFK_GEMM_TN && p->layout != CFK_GEMM_NN)
+    return fail(CFK_ERR_INVALID_ARG, "unknown GEMM layout %d", p->layout);
+  if (p->dtype == CFK_FP32 && p->layout != CFK_GEMM_TN)
+    return fail(CFK_ERR_UNSUPPORTED, "fp32 GEMM is built for the TN layout only");
+  if (p->m % 256 || p->n % 256 || p->k % 64)
+    return fail(CFK_ERR_UNSUPPORTED, "M and N must be multiples of 256 and K of 64 (got %d, %d, %d)", p->m, p->n, p->k);
+  if (p->batch > 65535) return fail(CFK_ERR_UNSUPPORTED, "batch must be <= 65535 (got %d)", p->batch);
   int rc = check_device();
   if (rc != CFK_OK) return rc;
-  hipError_t e = cfk::launch_gemm_f16(M, N, K, A, B, C, layout, (hipStream_t)stream);
-  if (e == hipErrorNotSupported) return fail(CFK_ERR_UNSUPPORTED, "GEMM layout %d is not built", layout);
+  cfk::GemmArgs g{};
+  g.A = p->a;
+  g.B = p->b;
+  g.C = p->c;
+  g.D = p->d;
+  g.M = p->m;
+  g.N = p->n;
+  g.K = p->k;
+  g.batch = p->batch;
+  g.layout = p->layout;
+  g.f32 = p->dtype == CFK_FP32;
+  g.alpha = p->alpha;
+  g.beta = p->beta;
+  hipError_t e = cfk::launch_gemm(g, (hipStream_t)stream);
+  if (e == hipErrorNotSupported) return fail(CFK_ERR_UNSUPPORTED, "GEMM dtype %d / layout %d is not built", p->dtype, p->layout);
   if (e != hipSuccess) return fail(CFK_ERR_HIP, "GEMM launch failed: %s", hipGetErrorString(e));
   return CFK_OK;
+}
+
+int cfk_gemm_f16(int32_t M, int32_t N, int32_t K, const void *A, const void *B, void *C, int32_t layout, void *stream) {
+  if (!C) return fail(CFK_ERR_INVALID_ARG, "A, B, C must be non-NULL device pointers");
+  cfk_gemm_params p{};
+  p.dtype = CFK_FP16;
+  p.layout = layout;
+  p.m = M;
+  p.n = N;
+  p.k = K;
+  p.batch = 1;
+  p.alpha = 1.0f;
+  p.beta = 0.0f;
+  p.a = A;
+  p.b = B;
+  p.c = nullptr;
+  p.d = C;
+  return cfk_gemm(&p, stream);
 }
 
 const char *cfk_last_error(void) { return g_err; }

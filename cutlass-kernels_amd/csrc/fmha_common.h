@@ -35,7 +35,15 @@ bool plan_fmha_f16(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *
 bool plan_fmha_fp8(int head_dim, int sq, int skv, int bh, int v_layout, bool tap_s, FmhaPlan *p);
 bool plan_fmha_hybrid(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *p);
 
-hipError_t launch_gemm_f16(int M, int N, int K, const void *A, const void *B, void *C, int layout, hipStream_t s);
+// D = alpha * A.B + beta * C for `batch` packed problems; f32 selects float operands (layout 0 only), else fp16.
+struct GemmArgs {
+  const void *A, *B, *C;  // C may be null (beta is then ignored)
+  void *D;
+  int32_t M, N, K, batch, layout;
+  bool f32;
+  float alpha, beta;
+};
+hipError_t launch_gemm(const GemmArgs &g, hipStream_t s);
 
 // Workgroup id -> logical tile id.  Hardware deals consecutive workgroup ids round-robin over the 8 XCDs,
 // each with a private L2.  Giving XCD x the contiguous range [x*n/8, (x+1)*n/8) keeps the query blocks

@@ -1,11 +1,14 @@
-// Dense GEMM C = A.B, fp16 operands, fp32 accumulate, fp16 C (row-major M x N) -- gfx950 only.
+// Dense (batched) GEMM D = alpha * A.B + beta * C with fp32 accumulation and an fp32 epilogue, D row-major M x N, for
+// fp16 operands (v_mfma_f32_32x32x16_f16) and fp32 operands (v_mfma_f32_32x32x2_f32) -- gfx950 only.
 //
-// Secondary bench on the FMHA tile engine: the same LDS-DMA staging with XOR-swizzled rows, the same
-// v_mfma_f32_32x32x16_f16 tiles.  Takes the place of gemm_device/gemm of the reference's CuTe example
-// (src/cute-gemm-tma-gma/gemm.cu:57-463: TMA load of one A and one B tile, one synchronous WGMMA batch per K-tile,
-// no pipelining).  Layouts: TN = A is M x K and B is N x K, both K-contiguous (the reference's form, :362-380);
-// NN = B is K x N, N-contiguous (the literal C = A.B), whose B operand is read with ds_read_b64_tr_b16 exactly as V
-// is in the attention kernel.  The reference writes C column-major (:386-389); C is row-major here.
+// Secondary bench on the FMHA tile engine: the same LDS-DMA staging with XOR-swizzled rows and 32x32 MFMA tiles.
+// Takes the place of gemm_device/gemm of the reference's CuTe example (src/cute-gemm-tma-gma/gemm.cu:57-463: TMA load
+// of one A and one B tile, one synchronous WGMMA batch per K-tile, no pipelining; its type 1 is float, type 3 half,
+// :677-684; batch count L with packed strides, :519-521) and of the CUTLASS-API example with its alpha / beta
+// epilogue (src/cutlass-gemm/gemm.cu:87-140, 318-324).  Layouts: TN = A is M x K and B is N x K, both K-contiguous
+// (the reference's form, :362-380); NN (fp16 only) = B is K x N, N-contiguous (the literal C = A.B), whose B operand is
+// read with ds_read_b64_tr_b16 exactly as V is in the attention kernel.  The reference writes C column-major
+// (:386-389); C and D are row-major here.  gfx950 has no tf32/xf32 MFMA: fp32 operands multiply in full fp32.
 //
 // Workgroup = 4 waves (one per SIMD) on a 256 x 256 macro tile; wave (wm, wn) of a 2 x 2 grid owns 128 x 128 of C as
 // 4 x 4 MFMA blocks, its 256 accumulator registers in the AGPR half of the register file.  K tiles are 32 deep and go
@@ -26,6 +29,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 256, BN = 256;
 
@@ -38,11 +42,17 @@ __device__ __forceinline__ int swz512(int row) { return (row & 3) << 2; }
 
 // WN = waves along n (2 along m always): 2 -> 4 waves of 128 x 128, one per SIMD (the shipped shape; a third less
 // LDS traffic per MFMA than 4 -> 8 waves of 128 x 64, two per SIMD).
-// BK = depth of a K tile, NS = LDS stages (copies run NS-1 tiles ahead of the multiply).
-template <bool NN, int WN, int BK, int NS>
+// T = element type of A, B, C, D (_Float16 or float); BKB = bytes of a K-contiguous tile row (32 halves or 16
+// floats at 64), NS = LDS stages (copies run NS-1 tiles ahead of the multiply).  blockIdx.y = problem of a batch.
+template <class T, bool NN, int WN, int BKB, int NS>
 __global__ void __launch_bounds__(2 * WN * 64) __attribute__((amdgpu_waves_per_eu(WN / 2, WN / 2)))
-gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, _Float16 *__restrict__ C, int M, int N,
-                int K) {
+gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restrict__ Cin, T *__restrict__ D, int M, int N,
+            int K, float alpha, float beta) {
+  constexpr bool F32 = sizeof(T) == 4;
+  constexpr int ES = sizeof(T);
+  constexpr int BK = BKB / ES;
+  static_assert(!(F32 && NN), "the N-contiguous B layout is built for fp16 only");
+  using Frag = std::conditional_t<F32, f32x4, half8>;  // 16 bytes of a row: the operand of one K-step
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -50,12 +60,12 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
   const int r = lane & 31, g = lane >> 5;
   constexpr int NWAVES = 2 * WN;
   constexpr int NB = BN / WN / 32;     // 32-column blocks per wave
-  constexpr int PITCH = BK * 2;        // bytes per K-contiguous LDS row
+  constexpr int PITCH = BKB;           // bytes per K-contiguous LDS row
   constexpr int A_TILE = BM * PITCH;   // TN: B tile likewise (n rows); NN: BK rows (k) of 512 B
   constexpr int STAGE = 2 * A_TILE;
   constexpr int CPW = A_TILE / 1024 / NWAVES;  // 1 KB copies per wave and operand tile
   constexpr int RPC = 1024 / PITCH;    // rows per copy
-  constexpr int KS = BK / 16;          // 16-deep K-steps per tile
+  constexpr int KS = PITCH / 32;       // K-steps per tile: 32 bytes of a row (one 16-byte fragment per lane half) each
   const int wm = wave / WN, wn = wave % WN;
 
   // tile order: groups of 8 tile rows, column-major inside a group, so concurrently running workgroups share A and
@@ -73,6 +83,11 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
   const int m0 = tm * BM, n0 = tn * BN;
 
   const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+  const int64_t batch = blockIdx.y;  // packed strides M*K, N*K, M*N (reference: gemm.cu:519-521)
+  A += batch * M * K;
+  B += batch * N * K;
+  D += batch * M * N;
+  if (Cin) Cin += batch * M * N;
   const char *Ap = (const char *)(A + (int64_t)m0 * K);
   const char *Bp = NN ? (const char *)(B + n0) : (const char *)(B + (int64_t)n0 * K);
 
@@ -83,7 +98,7 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
   for (int i = 0; i < CPW; ++i) {
     const int row = (i * NWAVES + wave) * RPC + lane / (PITCH / 16);
     const int cp = lane % (PITCH / 16);
-    goff_a[i] = (uint32_t)row * (uint32_t)(K * 2) + (uint32_t)((cp ^ swz_k<PITCH>(row)) * 16);
+    goff_a[i] = (uint32_t)row * (uint32_t)(K * ES) + (uint32_t)((cp ^ swz_k<PITCH>(row)) * 16);
     if (!NN) {
       goff_b[i] = goff_a[i];
     } else {  // B tile is BK rows (k) of 512 B (256 n): 2 rows per copy
@@ -93,15 +108,17 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
     }
   }
   auto load_stage = [&](int kt, int stage) {
-    const char *ga = Ap + (size_t)kt * (BK * 2);
-    const char *gb = NN ? Bp + (size_t)kt * BK * (size_t)(N * 2) : Bp + (size_t)kt * (BK * 2);
+    const char *ga = Ap + (size_t)kt * PITCH;
+    const char *gb = NN ? Bp + (size_t)kt * BK * (size_t)(N * 2) : Bp + (size_t)kt * PITCH;
 #pragma unroll
     for (int i = 0; i < CPW; ++i) lds_dma16(ga + goff_a[i], lds_base + stage * STAGE + (i * NWAVES + wave) * 1024);
 #pragma unroll
     for (int i = 0; i < CPW; ++i) lds_dma16(gb + goff_b[i], lds_base + stage * STAGE + A_TILE + (i * NWAVES + wave) * 1024);
   };
 
-  // ---- LDS read addresses.  K-step s (16 deep): lane (r, g) needs k = 16s + 8g .. +8 of its row.
+  // ---- LDS read addresses.  K-step s: lane (r, g) needs bytes 32s + 16g .. +16 of its row (fp16: k = 16s + 8g .. +8;
+  // fp32: k = 8s + 4g .. +4, used one element per 32x32x2 MFMA: which contraction slot means which k is free as long
+  // as A and B agree).
   int a_rd[KS], b_rd[KS];
 #pragma unroll
   for (int s = 0; s < KS; ++s) {
@@ -129,24 +146,26 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
 
   const int k_tiles = K / BK;
   // operand fetch for K-step s of the tile in LDS stage `st`
-  auto fetch = [&](const char *st, int s, half8 (&aop)[4], half8 (&bop)[NB]) {
+  auto fetch = [&](const char *st, int s, Frag (&aop)[4], Frag (&bop)[NB]) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       if (!NN) {
-        bop[nb] = *(const half8 *)(st + b_rd[s] + nb * 32 * PITCH);
+        bop[nb] = *(const Frag *)(st + b_rd[s] + nb * 32 * PITCH);
       } else {
-        union {
-          struct { short4v lo, hi; } p;
-          half8 h;
-        } u;
-        const char *bp = st + bt_rd[nb] + s * 16 * 512;
-        u.p.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp));
-        u.p.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp + 4 * 512));
-        bop[nb] = u.h;
+        if constexpr (!F32) {
+          union {
+            struct { short4v lo, hi; } p;
+            half8 h;
+          } u;
+          const char *bp = st + bt_rd[nb] + s * 16 * 512;
+          u.p.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp));
+          u.p.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp + 4 * 512));
+          bop[nb] = u.h;
+        }
       }
     }
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) aop[mb] = *(const half8 *)(st + a_rd[s] + mb * 32 * PITCH);
+    for (int mb = 0; mb < 4; ++mb) aop[mb] = *(const Frag *)(st + a_rd[s] + mb * 32 * PITCH);
   };
   // One copy (index c of the 2*CPW a wave issues per tile: first the A ones, then the B ones) of the tile at
   // ga / gb into stage `fill`
@@ -157,12 +176,19 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
   // The multiplies of one K-step, with the copies [c0, c1) of the tile being prefetched spread between them: the
   // L1 takes a 1 KB copy apart into sixteen 64-byte accesses, so copies issued back to back fill the memory
   // pipeline's queue and stall the wave (and with it the MFMA pipe) at the next one.
-  auto mma = [&](const half8 (&aop)[4], const half8 (&bop)[NB], const char *ga, const char *gb, int fill, int c0, int c1) {
+  auto mma = [&](const Frag (&aop)[4], const Frag (&bop)[NB], const char *ga, const char *gb, int fill, int c0, int c1) {
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)  // transposed block: MFMA rows = n (B operand first), columns = m
-        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop[mb], acc[mb][nb], 0, 0, 0);
+      for (int nb = 0; nb < NB; ++nb) {  // transposed block: MFMA rows = n (B operand first), columns = m
+        if constexpr (F32) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(bop[nb][e], aop[mb][e], acc[mb][nb], 0, 0, 0);
+        } else {
+          acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop[mb], acc[mb][nb], 0, 0, 0);
+        }
+      }
 #pragma unroll
       for (int c = c0 + mb; c < c1; c += 4) load_copy(ga, gb, fill, c);
       __builtin_amdgcn_sched_barrier(0);
@@ -180,7 +206,7 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
   for (int t0 = 0; t0 < NS - 1; ++t0) load_stage(t0 < k_tiles ? t0 : k_tiles - 1, t0);
   wait_lds_dma();
   __syncthreads();
-  half8 aop[2][4], bop[2][NB];  // two operand register sets: K-step s+1 is fetched while K-step s multiplies
+  Frag aop[2][4], bop[2][NB];  // two operand register sets: K-step s+1 is fetched while K-step s multiplies
   fetch(smem, 0, aop[0], bop[0]);
   int stage = 0;
   for (int kt = 0; kt < k_tiles; ++kt) {
@@ -188,8 +214,8 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
     // with tile kt+NS-1 (clamped at the end: a surplus copy rewrites a stage nobody reads any more)
     const int fill = stage == 0 ? NS - 1 : stage - 1;
     const int ld_t = kt + NS - 1 < k_tiles ? kt + NS - 1 : k_tiles - 1;
-    const char *ga = Ap + (size_t)ld_t * (BK * 2);
-    const char *gb = NN ? Bp + (size_t)ld_t * BK * (size_t)(N * 2) : Bp + (size_t)ld_t * (BK * 2);
+    const char *ga = Ap + (size_t)ld_t * PITCH;
+    const char *gb = NN ? Bp + (size_t)ld_t * BK * (size_t)(N * 2) : Bp + (size_t)ld_t * PITCH;
     const char *st = smem + stage * STAGE;
     const int nstage = stage + 1 == NS ? 0 : stage + 1;
     // sched_barrier(0): the compiler's scheduler would otherwise sink each fetch down to its first use and expose
@@ -210,41 +236,55 @@ gemm_f16_kernel(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, 
   }
   wait_lds_dma();  // no copy may still be writing LDS when the workgroup retires
 
-  // ---- epilogue: lane (m = r, g) holds n = 8i + 4g + j of each block
+  // ---- epilogue: D = alpha * acc + beta * C in fp32 (src/cutlass-gemm/gemm.cu:318-324); lane (m = r, g) holds
+  // n = 8i + 4g + j of each block: 4 consecutive elements of a row per access
+  using Out4 = std::conditional_t<F32, f32x4, half4>;
+  const bool with_c = Cin != nullptr && beta != 0.f;
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
-    _Float16 *crow = C + (int64_t)(m0 + wm * 128 + mb * 32 + r) * N + n0 + wn * NB * 32;
+    const int64_t row_off = (int64_t)(m0 + wm * 128 + mb * 32 + r) * N + n0 + wn * NB * 32;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        half4 o4;
+        const int64_t off = row_off + nb * 32 + 8 * i + 4 * g;
+        float v[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) o4[j] = (_Float16)acc[mb][nb][4 * i + j];
-        *(half4 *)(crow + nb * 32 + 8 * i + 4 * g) = o4;
+        for (int j = 0; j < 4; ++j) v[j] = alpha * acc[mb][nb][4 * i + j];
+        if (with_c) {
+          const Out4 c4 = *(const Out4 *)(Cin + off);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) v[j] += beta * (float)c4[j];
+        }
+        Out4 o4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o4[j] = (T)v[j];
+        *(Out4 *)(D + off) = o4;
       }
   }
 }
 
-template <bool NN, int WN, int BK, int NS>
-hipError_t launch(int M, int N, int K, const void *A, const void *B, void *C, hipStream_t s) {
+template <class T, bool NN>
+hipError_t launch(const GemmArgs &g, hipStream_t s) {
+  constexpr int WN = 2, BKB = 64, NS = 4;
   static bool attr_done = false;
-  auto kern = gemm_f16_kernel<NN, WN, BK, NS>;
-  constexpr int LDS_BYTES = NS * 2 * BM * BK * 2;
+  auto kern = gemm_kernel<T, NN, WN, BKB, NS>;
+  constexpr int LDS_BYTES = NS * 2 * BM * BKB;
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (e != hipSuccess) return e;
     attr_done = true;
   }
-  hipLaunchKernelGGL(kern, dim3((M / BM) * (N / BN)), dim3(2 * WN * 64), LDS_BYTES, s, (const _Float16 *)A, (const _Float16 *)B,
-                     (_Float16 *)C, M, N, K);
+  hipLaunchKernelGGL(kern, dim3((g.M / BM) * (g.N / BN), g.batch), dim3(2 * WN * 64), LDS_BYTES, s, (const T *)g.A,
+                     (const T *)g.B, (const T *)g.C, (T *)g.D, g.M, g.N, g.K, g.alpha, g.beta);
   return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t launch_gemm_f16(int M, int N, int K, const void *A, const void *B, void *C, int layout, hipStream_t s) {
-  return layout == 0 ? launch<false, 2, 32, 4>(M, N, K, A, B, C, s) : launch<true, 2, 32, 4>(M, N, K, A, B, C, s);
+hipError_t launch_gemm(const GemmArgs &g, hipStream_t s) {
+  if (g.f32) return g.layout == 0 ? launch<float, false>(g, s) : hipErrorNotSupported;
+  return g.layout == 0 ? launch<_Float16, false>(g, s) : launch<_Float16, true>(g, s);
 }
 
 }  // namespace cfk

@@ -17,6 +17,7 @@ _lib = None
 
 CFK_FP16 = 1
 CFK_FP8_E4M3 = 2
+CFK_FP32 = 3  # GEMM only
 CFK_V_BSHD = 0
 CFK_V_BDHS = 1
 CFK_GEMM_TN = 0
@@ -40,6 +41,16 @@ class FmhaFwdParams(ctypes.Structure):
         ("softmax_scale", ctypes.c_float),
         ("q_descale", ctypes.c_float), ("k_descale", ctypes.c_float), ("v_descale", ctypes.c_float),
         ("dbg_s", ctypes.c_void_p), ("dbg_row_max", ctypes.c_void_p), ("dbg_row_sum", ctypes.c_void_p),
+    ]
+
+
+class GemmParams(ctypes.Structure):
+    """``cfk_gemm_params`` (include/cfk_fmha.h)."""
+    _fields_ = [
+        ("dtype", ctypes.c_int32), ("layout", ctypes.c_int32),
+        ("m", ctypes.c_int32), ("n", ctypes.c_int32), ("k", ctypes.c_int32), ("batch", ctypes.c_int32),
+        ("alpha", ctypes.c_float), ("beta", ctypes.c_float),
+        ("a", ctypes.c_void_p), ("b", ctypes.c_void_p), ("c", ctypes.c_void_p), ("d", ctypes.c_void_p),
     ]
 
 
@@ -71,6 +82,8 @@ def lib():
         l.cfk_fmha_forward_plan.argtypes = [ctypes.POINTER(FmhaFwdParams)] + [ctypes.POINTER(ctypes.c_int32)] * 4
         l.cfk_gemm_f16.restype = ctypes.c_int
         l.cfk_gemm_f16.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p] * 3 + [ctypes.c_int32, ctypes.c_void_p]
+        l.cfk_gemm.restype = ctypes.c_int
+        l.cfk_gemm.argtypes = [ctypes.POINTER(GemmParams), ctypes.c_void_p]
         l.cfk_last_error.restype = ctypes.c_char_p
         l.cfk_version.restype = ctypes.c_char_p
         _lib = l
@@ -190,3 +203,39 @@ def gemm_f16(a, b, c=None, layout=CFK_GEMM_TN, stream=None):
         c = torch.empty((M, N), dtype=torch.float16, device=a.device)
     _check(lib().cfk_gemm_f16(M, N, K, a.data_ptr(), b.data_ptr(), c.data_ptr(), layout, _stream_ptr(stream)))
     return c
+
+
+def gemm(a, b, c=None, alpha=1.0, beta=0.0, out=None, layout=CFK_GEMM_TN, stream=None):
+    """D = alpha * A.B + beta * C, fp32 accumulate and epilogue (``cfk_gemm``).
+
+    ``a`` is [M,K] or [L,M,K]; ``b`` is [N,K] (TN, the reference's form, src/cute-gemm-tma-gma/gemm.cu:362-380) or
+    [K,N] (NN, fp16 only), with the same leading batch dimension; ``c`` / ``out`` are [M,N] or [L,M,N].  float16 or
+    float32 device tensors, all of one dtype (the reference's types 3 and 1, gemm.cu:677-684).
+    """
+    import torch
+    if a.dtype not in (torch.float16, torch.float32) or b.dtype != a.dtype or not (a.is_cuda and b.is_cuda):
+        raise ValueError("a, b must be float16 or float32 device tensors of one dtype")
+    if a.dim() not in (2, 3) or b.dim() != a.dim():
+        raise ValueError("a, b must both be 2-D or both 3-D (leading batch dimension)")
+    if not (a.is_contiguous() and b.is_contiguous()):
+        raise ValueError("a, b must be contiguous")
+    L = a.shape[0] if a.dim() == 3 else 1
+    M, K = a.shape[-2:]
+    N = b.shape[-2] if layout == CFK_GEMM_TN else b.shape[-1]
+    if tuple(b.shape[-2:]) != ((N, K) if layout == CFK_GEMM_TN else (K, N)) or (b.dim() == 3 and b.shape[0] != L):
+        raise ValueError("b shape mismatch")
+    shape = (L, M, N) if a.dim() == 3 else (M, N)
+    if out is None:
+        out = torch.empty(shape, dtype=a.dtype, device=a.device)
+    for t in (c, out):
+        if t is not None and (t.dtype != a.dtype or tuple(t.shape) != shape or not t.is_contiguous() or not t.is_cuda):
+            raise ValueError("c / out must be contiguous device tensors of a's dtype and shape " + str(shape))
+    p = GemmParams()
+    p.dtype = CFK_FP16 if a.dtype == torch.float16 else CFK_FP32
+    p.layout = layout
+    p.m, p.n, p.k, p.batch = M, N, K, L
+    p.alpha, p.beta = float(alpha), float(beta)
+    p.a, p.b, p.d = a.data_ptr(), b.data_ptr(), out.data_ptr()
+    p.c = c.data_ptr() if c is not None else None
+    _check(lib().cfk_gemm(ctypes.byref(p), _stream_ptr(stream)))
+    return out

@@ -33,7 +33,7 @@ typedef enum cfk_status {
 } cfk_status;
 
 /* Operand precision; values mirror the driver flag --prec-type (src/fmha-pipeline/fmha_forward.cu:694,733). */
-typedef enum cfk_dtype { CFK_FP16 = 1, CFK_FP8_E4M3 = 2 } cfk_dtype;
+typedef enum cfk_dtype { CFK_FP16 = 1, CFK_FP8_E4M3 = 2, CFK_FP32 = 3 /* GEMM only */ } cfk_dtype;
 
 /* Layout of V in memory. */
 typedef enum cfk_v_layout {
@@ -100,6 +100,26 @@ typedef enum cfk_gemm_layout {
  * M, N multiples of 256; K a multiple of 64. */
 int cfk_gemm_f16(int32_t M, int32_t N, int32_t K, const void *A, const void *B, void *C, int32_t layout,
                  void *stream);
+
+/* General form: D = alpha * A.B + beta * C for `batch` problems stored back to back (strides M*K, N*K, M*N elements).
+ * Replaces
+ *   - gemm(m, n, k, alpha, A, ldA, B, ldB, beta, C, ldC, ..., L) of the CuTe example
+ *     (src/cute-gemm-tma-gma/gemm.cu:336-463; type 1 = float operands, type 3 = half, :677-684; batch L, :519-521), and
+ *   - Gemm::Arguments{{m,n,k}, {A, B}, {{alpha, beta}, C, D}} of the CUTLASS-API example
+ *     (src/cutlass-gemm/gemm.cu:318-324).
+ * dtype = CFK_FP16 or CFK_FP32 is the element type of A, B, C and D; accumulation and the epilogue are fp32 (the
+ * reference accumulates in the C type).  gfx950 has no tf32 MFMA: CFK_FP32 multiplies in full fp32.  C and D are
+ * row-major M x N; c may be NULL (beta is then ignored) and may alias d.  CFK_GEMM_NN exists for CFK_FP16 only.
+ * M, N multiples of 256; K a multiple of 64; batch >= 1. */
+typedef struct cfk_gemm_params {
+  int32_t dtype;  /* cfk_dtype */
+  int32_t layout; /* cfk_gemm_layout */
+  int32_t m, n, k, batch;
+  float alpha, beta;
+  const void *a, *b, *c;
+  void *d;
+} cfk_gemm_params;
+int cfk_gemm(const cfk_gemm_params *p, void *stream);
 
 /* Message for the calling thread's most recent non-zero return ("" if none). */
 const char *cfk_last_error(void);

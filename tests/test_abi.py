@@ -17,7 +17,7 @@ def _declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = _declared_functions()
-    assert {"cfk_fmha_forward", "cfk_fmha_forward_plan", "cfk_gemm_f16", "cfk_last_error", "cfk_version"} <= set(names)
+    assert {"cfk_fmha_forward", "cfk_fmha_forward_plan", "cfk_gemm", "cfk_gemm_f16", "cfk_last_error", "cfk_version"} <= set(names)
     lib = ctypes.CDLL(pkg.lib_path())
     for n in names:
         assert getattr(lib, n) is not None, n
@@ -68,6 +68,19 @@ def test_error_paths_mirror_reference_driver():
     assert lib.cfk_fmha_forward_plan(ctypes.byref(p), None, None, None, None) == -1
     assert lib.cfk_gemm_f16(100, 256, 64, None, None, None, 0, None) == -1
     assert lib.cfk_gemm_f16(100, 256, 64, 1, 1, 1, 0, None) == -2
+    # cfk_gemm: argument checks come before any GPU work
+    assert lib.cfk_gemm(None, None) == -1
+    g = pkg.fmha.GemmParams()
+    assert ctypes.sizeof(g) == 8 * 4 + 4 * 8   # six int32, two floats, four pointers
+    g.dtype, g.layout, g.m, g.n, g.k, g.batch, g.a, g.b, g.d = pkg.CFK_FP32, 0, 256, 256, 64, 1, 1, 1, 1
+    g.dtype = 2                                 # e4m3 is not a GEMM type
+    assert lib.cfk_gemm(ctypes.byref(g), None) == -1
+    g.dtype, g.layout = pkg.CFK_FP32, 1         # fp32 has the TN layout only
+    assert lib.cfk_gemm(ctypes.byref(g), None) == -2
+    g.layout, g.k = 0, 100
+    assert lib.cfk_gemm(ctypes.byref(g), None) == -2
+    g.k, g.batch = 64, 0
+    assert lib.cfk_gemm(ctypes.byref(g), None) == -1
 
 
 def test_python_binding_refuses_cpu_tensors():

@@ -87,8 +87,11 @@ GEMM_DRIVER = os.path.join(ROOT, "cutlass-kernels_amd", "driver", "gemm")
 
 
 def test_gemm_driver_rejects_other_types():
-    r = subprocess.run([GEMM_DRIVER, "1"], capture_output=True, text=True, timeout=60)
+    # type 2 (tf32) is commented out in the reference as well (src/cute-gemm-tma-gma/gemm.cu:679-681)
+    r = subprocess.run([GEMM_DRIVER, "2"], capture_output=True, text=True, timeout=60)
     assert r.returncode != 0 and "invalid type value" in r.stdout
+    r = subprocess.run([GEMM_DRIVER, "--help"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0 and "--alpha" in r.stdout
 
 
 @pytest.mark.gpu
@@ -97,3 +100,21 @@ def test_gemm_driver_runs_and_checks():
     assert r.returncode == 0, r.stdout + r.stderr
     assert "CUTE_GEMM:" in r.stdout and "GFlop/s" in r.stdout and "L = 2" in r.stdout
     assert r.stdout.count("Passed") == 2 and "Failed" not in r.stdout
+
+
+@pytest.mark.gpu
+def test_gemm_driver_float_type():
+    # type 1 of the CuTe example: float operands (gemm.cu:677-678)
+    r = subprocess.run([GEMM_DRIVER, "1", "512", "256", "256", "1", "check"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "CUTE_GEMM:" in r.stdout and r.stdout.count("Passed") == 2 and "Failed" not in r.stdout
+
+
+@pytest.mark.gpu
+def test_gemm_driver_cutlass_example_options():
+    # the CUTLASS-API example's command line and report (src/cutlass-gemm/gemm.cu:198-236, 390-413)
+    r = subprocess.run([GEMM_DRIVER, "--m=1024", "--n=512", "--k=1024", "--alpha=2", "--beta=0.5", "--iterations=5"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "Disposition: Passed" in r.stdout and "Problem Size: 1024x512x1024" in r.stdout
+    assert "Avg runtime:" in r.stdout and "GFLOPS:" in r.stdout

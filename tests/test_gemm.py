@@ -1,4 +1,4 @@
-"""GPU parity of the dense fp16 GEMM (secondary bench, same tile engine) against the CPU oracle.
+"""GPU parity of the dense GEMM (secondary bench, same tile engine) against the CPU oracle.
 The reference checks its GEMM examples by equality on integer-valued inputs
 (src/cutlass-gemm/gemm.cu:277-294, 329-359; src/cute-gemm-tma-gma/gemm.cu:645-651); so does this."""
 import numpy as np
@@ -54,9 +54,52 @@ def test_config5_row_sample():
     np.testing.assert_allclose(got, want, rtol=2e-3, atol=1e-2)
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_alpha_beta_batch_integer_inputs_bit_exact(dtype):
+    # the CUTLASS-API example's run: D = alpha * A.B + beta * C on integer-valued operands in [-8, 8], checked for
+    # EQUALITY (src/cutlass-gemm/gemm.cu:277-294, 318-359); plus the CuTe example's batch count L (gemm.cu:519-521).
+    # Everything is an integer below 2^24 in fp32, so alpha = 2, beta = -3 keep the result exact before the final
+    # rounding to the output type.
+    import torch
+    L, M, N, K = 3, 256, 512, 192
+    rng = np.random.default_rng(17)
+    a = rng.integers(-8, 9, (L, M, K)).astype(np.float32)
+    b = rng.integers(-8, 9, (L, N, K)).astype(np.float32)
+    c = rng.integers(-8, 9, (L, M, N)).astype(np.float32)
+    want = np.stack([2.0 * oracle.gemm_f32(a[i], b[i]) - 3.0 * c[i] for i in range(L)]).astype(dtype)
+    got = pkg.gemm(to_dev(a.astype(dtype)), to_dev(b.astype(dtype)), c=to_dev(c.astype(dtype)), alpha=2.0, beta=-3.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), want)
+    # beta = 0 must not read C (NaNs there would otherwise leak), and D may alias C
+    cn = to_dev(np.full((L, M, N), np.nan, dtype))
+    got = pkg.gemm(to_dev(a.astype(dtype)), to_dev(b.astype(dtype)), c=cn, alpha=1.0, beta=0.0, out=cn)
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy(), np.stack([oracle.gemm_f32(a[i], b[i]) for i in range(L)]).astype(dtype))
+
+
+def test_fp32_uniform_inputs():
+    # the CuTe example's type 1 (float operands, gemm.cu:677-684), U(-1,1) data (:482-485).  Both sides accumulate in
+    # fp32 in different orders: |error| <~ sqrt(K) * 2^-24 * |terms|
+    import torch
+    M, N, K = 512, 256, 4096
+    a = pkg.testbed.uniform((M, K), 5).astype(np.float32)
+    b = pkg.testbed.uniform((N, K), 6).astype(np.float32)
+    want = oracle.gemm_f32(a, b)
+    got = pkg.gemm(to_dev(a), to_dev(b))
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-4, atol=2e-4)
+    # pins the contraction-slot mapping of the fp32 path against a float64 product on a few rows
+    ref64 = a[:8].astype(np.float64) @ b.astype(np.float64).T
+    np.testing.assert_allclose(got[:8].cpu().numpy(), ref64, rtol=1e-4, atol=2e-4)
+
+
 def test_error_paths():
     import torch
     x = torch.zeros((100, 64), dtype=torch.float16, device="cuda:0")
     with pytest.raises(pkg.CfkError) as e:
         pkg.gemm_f16(x, x)
+    assert e.value.code == -2
+    xf = torch.zeros((256, 64), dtype=torch.float32, device="cuda:0")
+    with pytest.raises(pkg.CfkError) as e:      # the N-contiguous B layout is an fp16 layout
+        pkg.gemm(xf, torch.zeros((64, 256), dtype=torch.float32, device="cuda:0"), layout=1)
     assert e.value.code == -2
