@@ -22,10 +22,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-PEAK_TFLOPS = {"f16": 2500.0, "f8": 5000.0}   # MI355X published dense MFMA peaks
+PEAK_TFLOPS = {"f16": 2500.0, "f8": 5000.0, "f32": 157.3}   # MI355X published dense MFMA peaks
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the same
 # counter reads for a plain 256 MiB copy: FETCH x2.0, WRITE x1.0); summaries are under profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"cfg2": (196792 + 65550) * 1024, "cfg4": (98464 + 65544) * 1024}
+MEASURED_TRAFFIC_BYTES = {"cfg2": (196792 + 65570) * 1024, "cfg4": (98460 + 65536) * 1024}
 
 WORKLOADS = {
     "cfg1": dict(kind="fmha", dtype="f16", B=1, H=8, S=512, D=64, scale=0.125),
@@ -33,6 +33,7 @@ WORKLOADS = {
     "cfg3": dict(kind="fmha", dtype="f16", B=2, H=8, S=8192, D=256, scale=None),
     "cfg4": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None),
     "cfg5": dict(kind="gemm", dtype="f16", M=8192, N=8192, K=8192),
+    "gemm_f32": dict(kind="gemm", dtype="f32", M=8192, N=8192, K=8192, max_steps=50),  # the CuTe example's type 1
 }
 NAMES = {
     "cfg1": "fmha_fwd fp16 B=1 H=8 S=512 D=64 non-causal",
@@ -40,6 +41,7 @@ NAMES = {
     "cfg3": "fmha_fwd fp16 B=2 H=8 S=8192 D=256 non-causal",
     "cfg4": "fmha_fwd fp8-e4m3 B=4 H=16 S=4096 D=128 non-causal, per-tensor amax scales, V [B,S,H,D]",
     "cfg5": "gemm fp16 M=N=K=8192 TN fp32-accumulate",
+    "gemm_f32": "gemm fp32 M=N=K=8192 TN (fp32 MFMA: gfx950 has no tf32)",
 }
 
 
@@ -92,16 +94,17 @@ def _make_gemm(pkg, w, seed=3080):
     import torch
     dev = torch.device("cuda:0")
     g = torch.Generator(device=dev).manual_seed(seed)
-    a = (torch.rand((w["M"], w["K"]), generator=g, device=dev) * 2 - 1).half()
-    b = (torch.rand((w["N"], w["K"]), generator=g, device=dev) * 2 - 1).half()
-    c = torch.empty((w["M"], w["N"]), dtype=torch.float16, device=dev)
-    return (lambda: pkg.gemm_f16(a, b, c=c)), 2.0 * w["M"] * w["N"] * w["K"], (a, b, c)
+    dt = torch.float16 if w["dtype"] == "f16" else torch.float32
+    a = (torch.rand((w["M"], w["K"]), generator=g, device=dev) * 2 - 1).to(dt)
+    b = (torch.rand((w["N"], w["K"]), generator=g, device=dev) * 2 - 1).to(dt)
+    c = torch.empty((w["M"], w["N"]), dtype=dt, device=dev)
+    return (lambda: pkg.gemm(a, b, out=c)), 2.0 * w["M"] * w["N"] * w["K"], (a, b, c)
 
 
 def run_workload(pkg, name, steps, warmup):
     w = WORKLOADS[name]
     fn, flop, keep = (_make_fmha if w["kind"] == "fmha" else _make_gemm)(pkg, w)
-    ms, wall_ms = _time_launches(fn, steps, warmup)
+    ms, wall_ms = _time_launches(fn, min(steps, w.get("max_steps", steps)), warmup)
     tflops = flop / (ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[w["dtype"]]
     return dict(workload=NAMES[name], ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, flop_per_step=flop,
