@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """FMHA-forward benchmark on one MI355X: prints ONE JSON line.
 
-Headline workload (BASELINE config 2): fp16, B=8 H=16 S=2048 D=128, non-causal, Q/K/V iid N(0,1) synthetic, fp32
+Headline workload (benchmark configuration 2): fp16, B=8 H=16 S=2048 D=128, non-causal, Q/K/V iid N(0,1) synthetic, fp32
 softmax/accumulate, fp16 output.  A "step" is one forward call over the whole batch through the C-ABI
 (``cfk_fmha_forward``), inputs resident in HBM.  FLOP = 4*B*H*Sq*Skv*D per step
 (src/fmha-pipeline/fmha_forward.cu:572-573); timing protocol = the reference's: warm-up launches, then the mean of
@@ -148,7 +148,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build is single-GPU (one MI355X); --gpus must be 1. "
-                 "Batch x heads shard without communication, see DESIGN.md.")
+                 "(batch, head) problems are independent: shard them over GPUs without communication.")
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")

@@ -32,7 +32,7 @@ def _check_full(B, S, H, D, kind="gaussian", seqlen_kv=None, scale=None):
 
 
 def test_config1_full_check():
-    # BASELINE config 1: B=1 H=8 S=512 D=64, scale 1/sqrt(64), full CPU check
+    # benchmark configuration 1: B=1 H=8 S=512 D=64, scale 1/sqrt(64), full CPU check
     _check_full(1, 512, 8, 64, scale=1.0 / 8.0)
 
 
@@ -152,10 +152,10 @@ def _subset_check(B, S, H, D):
 
 
 def test_config2_headline_shape_subset_check():
-    # BASELINE config 2: B=8 H=16 S=2048 D=128; four full (b,h) slices + every 61st row of every head
+    # benchmark configuration 2: B=8 H=16 S=2048 D=128; four full (b,h) slices + every 61st row of every head
     _subset_check(8, 2048, 16, 128)
 
 
 def test_config3_long_sequence_large_head_subset_check():
-    # BASELINE config 3: B=2 H=8 S=8192 D=256
+    # benchmark configuration 3: B=2 H=8 S=8192 D=256
     _subset_check(2, 8192, 8, 256)

@@ -229,7 +229,7 @@ def test_unsupported_modes_report_errors():
 
 
 def test_config4_subset_check():
-    # BASELINE config 4: fp8 e4m3 B=4 H=16 S=4096 D=128, per-tensor amax scales, V in [B,S,H,D]
+    # benchmark configuration 4: fp8 e4m3 B=4 H=16 S=4096 D=128, per-tensor amax scales, V in [B,S,H,D]
     B, S, H, D = 4, 4096, 16, 128
     q, k, v = pkg.testbed.qkv(B, S, H, D)
     got, (qf, kf, vf) = _run(q, k, v)

@@ -40,7 +40,7 @@ def test_uniform_inputs(layout):
 
 
 def test_config5_row_sample():
-    # BASELINE config 5: M=N=K=8192, U(-1,1) fp16, fp32 accumulate, fp16 C; 24 sampled rows against the oracle
+    # benchmark configuration 5: M=N=K=8192, U(-1,1) fp16, fp32 accumulate, fp16 C; 24 sampled rows against the oracle
     import torch
     M = N = K = 8192
     a = pkg.testbed.uniform((M, K), 3).astype(np.float16)
