@@ -180,6 +180,22 @@ def test_e4m3_decode_table_closed_form_and_torch():
     assert np.array_equal(np.nan_to_num(t, nan=12345.0), np.nan_to_num(table, nan=12345.0))
 
 
+def test_e4m3_codec_against_committed_fixture():
+    # tests/golden/e4m3_fixture.npz (written by tests/golden/make_e4m3_fixture.py from torch.float8_e4m3fn): every
+    # code's value, and the encoding of every rounding midpoint, its float32 neighbours, saturating values and
+    # random samples over 16 binades, both signs
+    import os
+    f = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "e4m3_fixture.npz"))
+    got = oracle.e4m3_decode(np.arange(256, dtype=np.uint8))
+    assert np.array_equal(np.isnan(got), np.isnan(f["decode"]))
+    assert np.array_equal(got[~np.isnan(got)], f["decode"][~np.isnan(got)])
+    enc = oracle.e4m3_encode(f["x"])
+    # -0.0 and +0.0 are one value; compare codes through their decoded values there
+    same = enc == f["codes"]
+    zero = (f["x"] == 0) | ((enc & 0x7F) == 0)
+    assert np.all(same | (zero & ((f["codes"] & 0x7F) == 0)))
+
+
 def test_e4m3_encode_rne_saturating_all_midpoints():
     table = oracle.e4m3_decode_table()
     pos = table[:0x7F].astype(np.float64)
