@@ -18,6 +18,7 @@
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef int int8v __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define HIP_CHECK(x)                                                                         \
   do {                                                                                       \
@@ -28,12 +29,16 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
     }                                                                                        \
   } while (0)
 
-// FP8 = false: fp16 32x32x16; true: e4m3 32x32x64.  `data` holds 4096 operand dwords per variant.
-template <bool FP8>
+// FP8 = false: fp16 32x32x16 (SMALL: 16x16x32); true: e4m3 32x32x64 (SMALL: 16x16x128).  The small shapes do half
+// the FLOP per instruction in half the passes.  `data` holds 4096 operand dwords per variant.
+template <bool FP8, bool SMALL>
 __global__ void __launch_bounds__(256) mfma_loop(float *out, int iters, long long *clk, const int *data) {
   f32x16 c[4];
+  f32x4 c4[8];  // eight independent chains: the 4-pass shapes have twice the issue rate per dependent chain
   for (int i = 0; i < 4; ++i)
     for (int v = 0; v < 16; ++v) c[i][v] = 0.f;
+  for (int i = 0; i < 8; ++i)
+    for (int v = 0; v < 4; ++v) c4[i][v] = 0.f;
   int8v a[4], b[4];
   for (int u = 0; u < 4; ++u)
     for (int t = 0; t < 8; ++t) {
@@ -45,12 +50,16 @@ __global__ void __launch_bounds__(256) mfma_loop(float *out, int iters, long lon
 #pragma unroll
     for (int u = 0; u < 16; ++u) {
       if (FP8) {
-        c[u % 4] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[u % 4], b[(u + 1) % 4], c[u % 4], 0, 0, 0, 0, 0, 0);
+        if (SMALL)
+          c4[u % 8] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[u % 4], b[(u + 1) % 4], c4[u % 8], 0, 0, 0, 0, 0, 0);
+        else
+          c[u % 4] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[u % 4], b[(u + 1) % 4], c[u % 4], 0, 0, 0, 0, 0, 0);
       } else {
         half8 ha, hb;
         __builtin_memcpy(&ha, &a[u % 4], 16);
         __builtin_memcpy(&hb, &b[(u + 1) % 4], 16);
-        c[u % 4] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ha, hb, c[u % 4], 0, 0, 0);
+        if (SMALL) c4[u % 8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ha, hb, c4[u % 8], 0, 0, 0);
+        else c[u % 4] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ha, hb, c[u % 4], 0, 0, 0);
       }
     }
   }
@@ -58,6 +67,8 @@ __global__ void __launch_bounds__(256) mfma_loop(float *out, int iters, long lon
   float s = 0.f;
   for (int i = 0; i < 4; ++i)
     for (int v = 0; v < 16; ++v) s += c[i][v];
+  for (int i = 0; i < 8; ++i)
+    for (int v = 0; v < 4; ++v) s += c4[i][v];
   if (s == 12345.678f) out[0] = s;  // keeps the loop alive
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     clk[0] = t1 - t0;
@@ -80,14 +91,14 @@ static uint8_t e4m3_of(float x) {  // coarse encoder, good enough for operand st
   return sign | (uint8_t)((exp << 3) | mant);
 }
 
-template <bool FP8>
+template <bool FP8, bool SMALL = false>
 static int measure(const char *label, const int *ddata, double target_ms, int cus) {
   float *dout;
   long long *dclk;
   HIP_CHECK(hipMalloc(&dout, 4));
   HIP_CHECK(hipMalloc(&dclk, 16));
   const int grid = cus * 2;  // two 4-wave workgroups per CU = two waves per SIMD
-  const double flop_per_mfma = FP8 ? 2.0 * 32 * 32 * 64 : 2.0 * 32 * 32 * 16;
+  const double flop_per_mfma = (FP8 ? 2.0 * 32 * 32 * 64 : 2.0 * 32 * 32 * 16) / (SMALL ? 2 : 1);
   int iters = 2000;
   hipEvent_t e0, e1;
   HIP_CHECK(hipEventCreate(&e0));
@@ -95,7 +106,7 @@ static int measure(const char *label, const int *ddata, double target_ms, int cu
   float ms = 0.f;
   for (int pass = 0; pass < 3; ++pass) {  // pass 0 sizes the run, pass 1 settles the clock, pass 2 is reported
     HIP_CHECK(hipEventRecord(e0));
-    hipLaunchKernelGGL(mfma_loop<FP8>, dim3(grid), dim3(256), 0, 0, dout, iters, dclk, ddata);
+    hipLaunchKernelGGL((mfma_loop<FP8, SMALL>), dim3(grid), dim3(256), 0, 0, dout, iters, dclk, ddata);
     HIP_CHECK(hipEventRecord(e1));
     HIP_CHECK(hipEventSynchronize(e1));
     HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
@@ -143,6 +154,11 @@ int main(int argc, char **argv) {
   if (measure<false>("fp16 32x32x16, N(0,1) operands", d + 4096, target_ms, cus)) return 2;
   if (measure<true>("fp8 e4m3 32x32x64, constant operands", d + 8192, target_ms, cus)) return 2;
   if (measure<true>("fp8 e4m3 32x32x64, N(0,1)*64 operands", d + 12288, target_ms, cus)) return 2;
+  if (measure<false>("fp16 32x32x16, N(0,1) operands (repeat)", d + 4096, target_ms, cus)) return 2;
+  if (measure<false, true>("fp16 16x16x32, constant operands", d, target_ms, cus)) return 2;
+  if (measure<false, true>("fp16 16x16x32, N(0,1) operands", d + 4096, target_ms, cus)) return 2;
+  if (measure<true, true>("fp8 e4m3 16x16x128, constant operands", d + 8192, target_ms, cus)) return 2;
+  if (measure<true, true>("fp8 e4m3 16x16x128, N(0,1)*64 operands", d + 12288, target_ms, cus)) return 2;
   if (measure<false>("fp16 32x32x16, N(0,1) operands (repeat)", d + 4096, target_ms, cus)) return 2;
   return 0;
 }
