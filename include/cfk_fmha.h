@@ -1,6 +1,6 @@
 /*
  * cfk_fmha.h -- C-ABI of libcfk_fmha.so: fused multi-head-attention forward (fp16 and fp8 e4m3) and the
- * dense fp16 GEMM example for AMD Instinct MI355X (gfx950).
+ * dense GEMM examples (fp16 / fp32 operands) for AMD Instinct MI355X (gfx950).
  *
  * The reference repository (ColfaxResearch/cutlass-kernels) has no FFI: its hot path sits behind the C++
  * template fmhaForwardDevice<PrecType, Gemm2Type, SoftType, OutputType, HEADDIM>
@@ -56,7 +56,7 @@ typedef struct cfk_fmha_fwd_params {
   int32_t batch;     /* BATCH                                                                                 */
   int32_t heads;     /* NUMHEADS                                                                              */
   int32_t seqlen_q;  /* SEQLEN: multiple of 128                                                               */
-  int32_t seqlen_kv; /* KEYLEN: multiple of 128                                                               */
+  int32_t seqlen_kv; /* KEYLEN: multiple of the key tile cfk_fmha_forward_plan reports (64; 32 for fp16 V at 256)   */
   int32_t head_dim;  /* HEADDIM: 64, 128 or 256 (fmha_forward.cu:746-761)                                     */
   int32_t v_layout;  /* cfk_v_layout                                                                          */
   const void *q;     /* [B, S_q,  H, D] dtype, D contiguous (fmha_forward.cu:151-152)                         */
