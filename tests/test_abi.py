@@ -59,6 +59,11 @@ def test_error_paths_mirror_reference_driver():
     with pytest.raises(pkg.CfkError):
         pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, 64, v_layout=1)
     pkg.fmha_forward_plan(pkg.CFK_FP8_E4M3, 1, 1, 512, 512, 128, v_layout=1)
+    # one batch entry is addressed with 32-bit byte offsets: S * H * D * 2 bytes must stay below 2 GiB
+    with pytest.raises(pkg.CfkError) as e:
+        pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 64, 131072, 131072, 128)
+    assert e.value.code == -2 and "2 GiB" in str(e.value)
+    pkg.fmha_forward_plan(pkg.CFK_FP16, 64, 16, 65536, 65536, 128)   # large batch is fine: entries are 64-bit apart
     # null params / null pointers
     lib = pkg.lib()
     assert lib.cfk_fmha_forward(None, None) == -1

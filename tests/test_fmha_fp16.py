@@ -46,6 +46,14 @@ def test_rectangular_q_kv():
     _check_full(2, 512, 2, 64, seqlen_kv=128)
 
 
+@pytest.mark.parametrize("B,S,H,D,Skv", [(1, 128, 1, 64, 64), (1, 128, 1, 128, 64), (2, 256, 2, 128, 192),
+                                         (1, 256, 3, 64, 320), (1, 128, 2, 256, 32), (1, 128, 2, 256, 96)])
+def test_shortest_and_odd_key_tile_counts(B, S, H, D, Skv):
+    # one key tile (the pipeline is prologue + last step only), an odd number of tiles (the loop's other tail), and
+    # the smallest problem the tiles allow: one workgroup, one (batch, head)
+    _check_full(B, S, H, D, seqlen_kv=Skv)
+
+
 def test_integer_valued_inputs():
     _check_full(1, 256, 2, 64, kind="uniform_int")
 

@@ -48,6 +48,11 @@ def test_shapes_per_tensor_scales(B, S, H, D):
     _check_full(B, S, H, D)
 
 
+@pytest.mark.parametrize("B,S,H,D,Skv", [(1, 128, 1, 64, 64), (1, 128, 1, 128, 64), (2, 256, 2, 128, 192), (1, 128, 2, 256, 64)])
+def test_shortest_and_odd_key_tile_counts(B, S, H, D, Skv):
+    _check_full(B, S, H, D, seqlen_kv=Skv)
+
+
 def test_reference_mode_unit_scales():
     _check_full(1, 512, 2, 128, per_tensor=False)
 
