@@ -156,6 +156,12 @@ int cfk_gemm(const cfk_gemm_params *p, void *stream) {
   if (p->m % 256 || p->n % 256 || p->k % 64)
     return fail(CFK_ERR_UNSUPPORTED, "M and N must be multiples of 256 and K of 64 (got %d, %d, %d)", p->m, p->n, p->k);
   if (p->batch > 65535) return fail(CFK_ERR_UNSUPPORTED, "batch must be <= 65535 (got %d)", p->batch);
+  // the kernel addresses a 256-row tile of A / B (TN) and a 64-row K-slab of B (NN) with 32-bit byte offsets
+  const long long esz = p->dtype == CFK_FP32 ? 4 : 2;
+  if (256LL * p->k * esz >= (1LL << 32))
+    return fail(CFK_ERR_UNSUPPORTED, "K too large: 256 * K * element size must stay below 4 GiB (K = %d)", p->k);
+  if (p->layout == CFK_GEMM_NN && 64LL * p->n * 2 >= (1LL << 32))
+    return fail(CFK_ERR_UNSUPPORTED, "N too large for the NN layout: 64 * N * 2 must stay below 4 GiB (N = %d)", p->n);
   int rc = check_device();
   if (rc != CFK_OK) return rc;
   cfk::GemmArgs g{};
@@ -195,8 +201,19 @@ int cfk_gemm_f16(int32_t M, int32_t N, int32_t K, const void *A, const void *B, 
   return cfk_gemm(&p, stream);
 }
 
+int cfk_init(void) {
+  int rc = check_device();
+  if (rc != CFK_OK) return rc;
+  hipError_t e = cfk::prepare_fmha_f16();
+  if (e == hipSuccess) e = cfk::prepare_fmha_fp8();
+  if (e == hipSuccess) e = cfk::prepare_fmha_hybrid();
+  if (e == hipSuccess) e = cfk::prepare_gemm();
+  if (e != hipSuccess) return fail(CFK_ERR_HIP, "kernel set-up failed: %s", hipGetErrorString(e));
+  return CFK_OK;
+}
+
 const char *cfk_last_error(void) { return g_err; }
 
-const char *cfk_version(void) { return "cfk-mi355x 0.1 gfx950"; }
+const char *cfk_version(void) { return "cfk-mi355x 0.2 gfx950"; }
 
 }  // extern "C"

@@ -34,6 +34,12 @@ hipError_t launch_fmha_hybrid(const FmhaArgs &a, int head_dim, hipStream_t s);  
 bool plan_fmha_f16(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *p);
 bool plan_fmha_fp8(int head_dim, int sq, int skv, int bh, int v_layout, bool tap_s, FmhaPlan *p);
 bool plan_fmha_hybrid(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *p);
+// One-time set-up (dynamic-LDS limits) of every instantiation of a family on the current device; launches do it on
+// demand, this makes it happen ahead of time.
+hipError_t prepare_fmha_f16();
+hipError_t prepare_fmha_fp8();
+hipError_t prepare_fmha_hybrid();
+hipError_t prepare_gemm();
 
 // D = alpha * A.B + beta * C for `batch` packed problems; f32 selects float operands (layout 0 only), else fp16.
 struct GemmArgs {
@@ -57,6 +63,8 @@ __device__ __forceinline__ int xcd_remap(int wg, int n) {
 }
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T *)(p))
+// LDS pointer from an absolute LDS byte address (32-bit integer)
+#define LDS_AT(T, addr) ((__attribute__((address_space(3))) T *)(uintptr_t)(addr))
 
 // Asynchronous 16 B/lane global -> LDS copy: lane l writes LDS bytes [lds_addr + 16 l, +16) with the 16 bytes at
 // its own global address.  Issued through inline asm on purpose: the compiler then does not track the copy, so it
@@ -68,6 +76,12 @@ __device__ __forceinline__ void lds_dma16(const void *gptr, uint32_t lds_addr) {
 // The same copy addressed as wave-uniform base (SGPR pair) + per-lane 32-bit byte offset: no 64-bit vector add per copy.
 __device__ __forceinline__ void lds_dma16(const void *base, uint32_t lane_off, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off), "s"(base) : "memory");
+}
+// ... and with the LDS address as the sum of two wave-uniform terms (a long-lived one, e.g. the wave's share of every
+// tile, plus one that is a constant at most call sites): keeps one scalar register live instead of one per target.
+__device__ __forceinline__ void lds_dma16(const void *base, uint32_t lane_off, uint32_t lds_a, uint32_t lds_b) {
+  asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" ::"s"(lds_a), "s"(lds_b), "v"(lane_off), "s"(base)
+               : "memory", "scc");
 }
 __device__ __forceinline__ void wait_lds_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

@@ -5,47 +5,58 @@
 namespace cfk {
 namespace {
 
-using Cfg64S = FmhaCfg<64, 64, 4, 3, true, true>;  // three waves per SIMD: the VALU-bound softmax gains from every extra wave
-using Cfg128S = FmhaCfg<128, 64, 4, 2, true, true>;
-using Cfg128L = FmhaCfg<128, 64, 8, 2, true, true>;
-using Cfg256S = FmhaCfg<256, 64, 4, 1, true, true>;  // O (128) + S (64) + Q (32) registers: one wave per SIMD
+// template arguments as in fmha_fwd_f16.hip.  Head dim 64 runs three waves per SIMD (the VALU-bound softmax gains from
+// every extra wave); head dim 256 one (O 128 + S 64 + Q 32 registers).
+using C64_128x64 = FmhaCfg<64, 64, 4, 3, true, true>;
+using C64_128x128 = FmhaCfg<64, 64, 4, 2, true, true, false, false, 2>;
+using C128_128x64 = FmhaCfg<128, 64, 4, 2, true, true>;
+using C128_256x64 = FmhaCfg<128, 64, 8, 2, true, true>;
+using C128_128x128 = FmhaCfg<128, 64, 4, 2, true, true, false, false, 2>;
+using C128_256x128 = FmhaCfg<128, 64, 8, 2, true, true, false, false, 2>;
+using C256_128x64 = FmhaCfg<256, 64, 4, 1, true, true>;
+using C256_128x128 = FmhaCfg<256, 64, 4, 1, true, true, false, false, 2>;
 
 // V pre-transposed to [B,D,H,S] (the reference's offline transpose, src/fmha-pipeline/fmha_forward.cu:514-532)
-using Cfg64T = FmhaCfg<64, 64, 4, 2, true, true, true>;
-using Cfg128T = FmhaCfg<128, 64, 4, 2, true, true, true>;
-using Cfg256T = FmhaCfg<256, 64, 4, 1, true, true, true>;
+using C64T = FmhaCfg<64, 64, 4, 2, true, true, true>;
+using C128T = FmhaCfg<128, 64, 4, 2, true, true, true>;
+using C256T = FmhaCfg<256, 64, 4, 1, true, true, true>;
 
 // builds that also write the score tap (debug)
-using Cfg64Tap = FmhaCfg<64, 64, 4, 2, true, true, false, true>;
-using Cfg128Tap = FmhaCfg<128, 64, 4, 2, true, true, false, true>;
-using Cfg256Tap = FmhaCfg<256, 64, 4, 1, true, true, false, true>;
-using Cfg64TTap = FmhaCfg<64, 64, 4, 2, true, true, true, true>;
-using Cfg128TTap = FmhaCfg<128, 64, 4, 2, true, true, true, true>;
-using Cfg256TTap = FmhaCfg<256, 64, 4, 1, true, true, true, true>;
+using C64Tap = FmhaCfg<64, 64, 4, 2, true, true, false, true>;
+using C128Tap = FmhaCfg<128, 64, 4, 2, true, true, false, true>;
+using C256Tap = FmhaCfg<256, 64, 4, 1, true, true, false, true>;
+using C64TTap = FmhaCfg<64, 64, 4, 2, true, true, true, true>;
+using C128TTap = FmhaCfg<128, 64, 4, 2, true, true, true, true>;
+using C256TTap = FmhaCfg<256, 64, 4, 1, true, true, true, true>;
+
+using All64 = CfgList<C64_128x64, C64_128x128>;
+using All128 = CfgList<C128_128x64, C128_256x64, C128_128x128, C128_256x128>;
+using All256 = CfgList<C256_128x64, C256_128x128>;
 
 template <class F>
-bool dispatch(int head_dim, int sq, int bh, int v_layout, bool tap_s, F &&f) {
+bool dispatch(int head_dim, int sq, int skv, int bh, int v_layout, bool tap_s, F &&f) {
   if (tap_s) {
     const bool t = v_layout == 1;
     switch (head_dim) {
-      case 64: t ? f(Cfg64TTap{}) : f(Cfg64Tap{}); return true;
-      case 128: t ? f(Cfg128TTap{}) : f(Cfg128Tap{}); return true;
-      case 256: t ? f(Cfg256TTap{}) : f(Cfg256Tap{}); return true;
+      case 64: t ? f(C64TTap{}) : f(C64Tap{}); return true;
+      case 128: t ? f(C128TTap{}) : f(C128Tap{}); return true;
+      case 256: t ? f(C256TTap{}) : f(C256Tap{}); return true;
       default: return false;
     }
   }
   if (v_layout == 1) {
     switch (head_dim) {
-      case 64: f(Cfg64T{}); return true;
-      case 128: f(Cfg128T{}); return true;
-      case 256: f(Cfg256T{}); return true;
+      case 64: f(C64T{}); return true;
+      case 128: f(C128T{}); return true;
+      case 256: f(C256T{}); return true;
       default: return false;
     }
   }
   switch (head_dim) {
-    case 64: f(Cfg64S{}); return true;
-    case 128: use_large_tile(sq, bh, false) ? f(Cfg128L{}) : f(Cfg128S{}); return true;
-    case 256: f(Cfg256S{}); return true;
+    case 64: select_tile<All64, CfgList<C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
+    // big problems: 256 rows with one barrier per 128 keys (+4 % on N(0,1) data over the 128x64 tile)
+    case 128: select_tile<All128, CfgList<C128_256x128, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
+    case 256: select_tile<All256, CfgList<C256_128x64>, C256_128x64>(sq, skv, bh, f); return true;
     default: return false;
   }
 }
@@ -53,13 +64,20 @@ bool dispatch(int head_dim, int sq, int bh, int v_layout, bool tap_s, F &&f) {
 }  // namespace
 
 bool plan_fmha_fp8(int head_dim, int sq, int skv, int bh, int v_layout, bool tap_s, FmhaPlan *p) {
-  (void)skv;
-  return dispatch(head_dim, sq, bh, v_layout, tap_s, [&](auto cfg) { fill_fmha_plan<decltype(cfg)>(sq, bh, p); });
+  return dispatch(head_dim, sq, skv, bh, v_layout, tap_s, [&](auto cfg) { fill_fmha_plan<decltype(cfg)>(sq, bh, p); });
 }
 
 hipError_t launch_fmha_fp8(const FmhaArgs &a, int head_dim, hipStream_t s) {
   hipError_t e = hipErrorNotSupported;
-  dispatch(head_dim, a.Sq, a.B * a.H, a.v_layout, a.s_tap != nullptr, [&](auto cfg) { e = launch_fmha_cfg<decltype(cfg)>(a, s); });
+  dispatch(head_dim, a.Sq, a.Skv, a.B * a.H, a.v_layout, a.s_tap != nullptr, [&](auto cfg) { e = launch_fmha_cfg<decltype(cfg)>(a, s); });
+  return e;
+}
+
+hipError_t prepare_fmha_fp8() {
+  hipError_t e = prepare_all(All64{});
+  if (e == hipSuccess) e = prepare_all(All128{});
+  if (e == hipSuccess) e = prepare_all(All256{});
+  if (e == hipSuccess) e = prepare_all(CfgList<C64T, C128T, C256T, C64Tap, C128Tap, C256Tap, C64TTap, C128TTap, C256TTap>{});
   return e;
 }
 

@@ -6,30 +6,37 @@
 namespace cfk {
 namespace {
 
-using Cfg64S = FmhaCfg<64, 64, 4, 3, true, false>;
-using Cfg128S = FmhaCfg<128, 64, 4, 2, true, false>;
-using Cfg128L = FmhaCfg<128, 64, 8, 2, true, false>;
-using Cfg256S = FmhaCfg<256, 32, 4, 1, true, false>;
+// template arguments as in fmha_fwd_f16.hip
+using C64_128x64 = FmhaCfg<64, 64, 4, 3, true, false>;
+using C64_128x128 = FmhaCfg<64, 64, 4, 2, true, false, false, false, 2>;
+using C128_128x64 = FmhaCfg<128, 64, 4, 2, true, false>;
+using C128_256x64 = FmhaCfg<128, 64, 8, 2, true, false>;
+using C128_256x128 = FmhaCfg<128, 64, 8, 2, true, false, false, false, 2>;
+using C256_128x32 = FmhaCfg<256, 32, 4, 1, true, false>;
 
-// builds that also write the score tap (debug): small tile only
-using Cfg64Tap = FmhaCfg<64, 64, 4, 2, true, false, false, true>;
-using Cfg128Tap = FmhaCfg<128, 64, 4, 2, true, false, false, true>;
-using Cfg256Tap = FmhaCfg<256, 32, 4, 1, true, false, false, true>;
+// builds that also write the score tap (debug): 128-row tile only
+using C64Tap = FmhaCfg<64, 64, 4, 2, true, false, false, true>;
+using C128Tap = FmhaCfg<128, 64, 4, 2, true, false, false, true>;
+using C256Tap = FmhaCfg<256, 32, 4, 1, true, false, false, true>;
+
+using All64 = CfgList<C64_128x64, C64_128x128>;
+using All128 = CfgList<C128_128x64, C128_256x64, C128_256x128>;
+using All256 = CfgList<C256_128x32>;
 
 template <class F>
-bool dispatch(int head_dim, int sq, int bh, bool tap_s, F &&f) {
+bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
   if (tap_s) {
     switch (head_dim) {
-      case 64: f(Cfg64Tap{}); return true;
-      case 128: f(Cfg128Tap{}); return true;
-      case 256: f(Cfg256Tap{}); return true;
+      case 64: f(C64Tap{}); return true;
+      case 128: f(C128Tap{}); return true;
+      case 256: f(C256Tap{}); return true;
       default: return false;
     }
   }
   switch (head_dim) {
-    case 64: f(Cfg64S{}); return true;
-    case 128: use_large_tile(sq, bh) ? f(Cfg128L{}) : f(Cfg128S{}); return true;
-    case 256: f(Cfg256S{}); return true;
+    case 64: select_tile<All64, CfgList<C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
+    case 128: select_tile<All128, CfgList<C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
+    case 256: select_tile<All256, CfgList<C256_128x32>, C256_128x32>(sq, skv, bh, f); return true;
     default: return false;
   }
 }
@@ -37,13 +44,20 @@ bool dispatch(int head_dim, int sq, int bh, bool tap_s, F &&f) {
 }  // namespace
 
 bool plan_fmha_hybrid(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *p) {
-  (void)skv;
-  return dispatch(head_dim, sq, bh, tap_s, [&](auto cfg) { fill_fmha_plan<decltype(cfg)>(sq, bh, p); });
+  return dispatch(head_dim, sq, skv, bh, tap_s, [&](auto cfg) { fill_fmha_plan<decltype(cfg)>(sq, bh, p); });
 }
 
 hipError_t launch_fmha_hybrid(const FmhaArgs &a, int head_dim, hipStream_t s) {
   hipError_t e = hipErrorNotSupported;
-  dispatch(head_dim, a.Sq, a.B * a.H, a.s_tap != nullptr, [&](auto cfg) { e = launch_fmha_cfg<decltype(cfg)>(a, s); });
+  dispatch(head_dim, a.Sq, a.Skv, a.B * a.H, a.s_tap != nullptr, [&](auto cfg) { e = launch_fmha_cfg<decltype(cfg)>(a, s); });
+  return e;
+}
+
+hipError_t prepare_fmha_hybrid() {
+  hipError_t e = prepare_all(All64{});
+  if (e == hipSuccess) e = prepare_all(All128{});
+  if (e == hipSuccess) e = prepare_all(All256{});
+  if (e == hipSuccess) e = prepare_all(CfgList<C64Tap, C128Tap, C256Tap>{});
   return e;
 }
 

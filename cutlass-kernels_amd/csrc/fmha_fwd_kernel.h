@@ -50,12 +50,15 @@
 //  * Per-tensor fp8 scales: q_descale*k_descale is folded into the exp2 scale, v_descale into the final 1/l.
 //  * Workgroup ids are remapped so the query blocks of one head share an XCD's L2.
 #pragma once
+#include <cstdio>
+#include <mutex>
 #include <type_traits>
 
 #include "fmha_common.h"
 
 namespace cfk {
 
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -65,9 +68,13 @@ typedef int int8v __attribute__((ext_vector_type(8)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int2v __attribute__((ext_vector_type(2)));
 
-template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_, bool VT_ = false, bool TAP_S_ = false>
+template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_, bool VT_ = false, bool TAP_S_ = false, int SUB_ = 1, int KPRE_ = 0>
 struct FmhaCfg {
   static constexpr int D = D_, BN = BN_, NWAVES = NWAVES_;
+  static constexpr int SUB = SUB_;                              // BN-key sub-tiles per barrier (1 or 2)
+  static constexpr int KPRE = KPRE_;                            // K fragments of the next step read before the barrier
+  static constexpr int NSLOT = KPRE ? 4 : 2 * SUB;              // LDS slots of one BN-key sub-tile of K
+  static constexpr int NSLOT_V = 2 * SUB;                       // ... and of V
   static constexpr int WPE = WPE_;                              // waves per SIMD the register budget is sized for
   static constexpr bool QK8 = QK8_, PV8 = PV8_;                 // e4m3 (true) or fp16 (false) operands of GEMM-I / II
   static constexpr bool VT = VT_;                               // V given pre-transposed, [B,D,H,S] (e4m3 only)
@@ -78,12 +85,17 @@ struct FmhaCfg {
   static constexpr int V_PITCH = VT ? BN : D * (PV8 ? 1 : 2);   // VT: the tile is [d][key], rows of BN bytes
   static constexpr int V_ROWS = VT ? D : BN;
   static constexpr int K_TILE = BN * K_PITCH, V_TILE = V_ROWS * V_PITCH;
-  static constexpr int K_ST0 = 0, V_ST0 = 2 * K_TILE;           // LDS map: K stage 0/1, V stage 0/1
-  static constexpr int LDS_BYTES = 2 * K_TILE + 2 * V_TILE;
+  static constexpr int K_ST0 = 0, V_ST0 = NSLOT * K_TILE;       // LDS map: K slots, then V slots
+  static constexpr int O_PITCH = D * 2 + 16;                    // epilogue: a wave's 32 fp16 output rows, padded
+  static constexpr int STAGE_BYTES = NSLOT * K_TILE + NSLOT_V * V_TILE;
+  static constexpr int O_BYTES = NWAVES * 32 * O_PITCH;
+  static constexpr int LDS_BYTES = STAGE_BYTES > O_BYTES ? STAGE_BYTES : O_BYTES;
   // one wave-wide 16 B/lane copy moves 1 KB = RPI rows; IPW copies per wave and tile
   static constexpr int K_RPI = 1024 / K_PITCH, K_IPW = BN / K_RPI / NWAVES;
   static constexpr int V_RPI = 1024 / V_PITCH, V_IPW = V_ROWS / V_RPI / NWAVES;
   static_assert(D == 64 || D == 128 || D == 256, "head dim");
+  static_assert(SUB == 1 || SUB == 2, "sub-tiles per barrier");
+  static_assert(!KPRE || SUB == 1, "K fragment prefetch is a variant of the one-tile step");
   static_assert(BN % 32 == 0 && (!PV8 || BN == 64), "key tile: the e4m3 second GEMM has 64-deep K-steps");
   static_assert(!VT || PV8, "the pre-transposed layout is an e4m3-V layout");
   static_assert(K_IPW >= 1 && K_IPW * K_RPI * NWAVES == BN && V_IPW >= 1 && V_IPW * V_RPI * NWAVES == V_ROWS,
@@ -176,17 +188,18 @@ fmha_fwd_kernel(const FmhaArgs a) {
     goff_v[i] = (uint32_t)row * v_ld + (uint32_t)(((lane % CPR) ^ sw) * 16);
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
+  const uint32_t lds_wave = lds_base + wave * 1024;  // this wave's 1 KB share of every copy group
   auto load_k = [&](int jt, int stage) {
     const char *gt = Kp + (size_t)jt * ((size_t)BN * k_ld);
 #pragma unroll
     for (int i = 0; i < C::K_IPW; ++i)
-      lds_dma16(gt, goff_k[i], lds_base + C::K_ST0 + stage * C::K_TILE + (i * C::NWAVES + wave) * 1024);
+      lds_dma16(gt, goff_k[i], lds_wave, C::K_ST0 + stage * C::K_TILE + i * C::NWAVES * 1024);
   };
   auto load_v = [&](int jt, int stage) {
     const char *gt = C::VT ? Vp + (size_t)jt * BN : Vp + (size_t)jt * ((size_t)BN * v_ld);
 #pragma unroll
     for (int i = 0; i < C::V_IPW; ++i)
-      lds_dma16(gt, goff_v[i], lds_base + C::V_ST0 + stage * C::V_TILE + (i * C::NWAVES + wave) * 1024);
+      lds_dma16(gt, goff_v[i], lds_wave, C::V_ST0 + stage * C::V_TILE + i * C::NWAVES * 1024);
   };
 
   // ---- Q: B operand of S^T, resident in VGPRs.  fp16: lane (r, g), K-step s holds Q[q0+r][16s + 8g .. +8);
@@ -204,21 +217,21 @@ fmha_fwd_kernel(const FmhaArgs a) {
     }
   }
 
-  // ---- per-lane LDS read addresses (bytes, relative to a tile)
+  // ---- per-lane LDS read addresses (absolute LDS byte addresses of slot 0; slots and sub-blocks are immediates)
   // K operand, K-step s: row r (+32 kb); fp16 chunk 2s+g, e4m3 chunks 4s+2g and 4s+2g+1 (each swizzled on its own)
-  int k_rd[KS][KH];
+  uint32_t k_rd[KS][KH];
 #pragma unroll
   for (int s = 0; s < KS; ++s)
 #pragma unroll
     for (int hh = 0; hh < KH; ++hh)
-      k_rd[s][hh] = r * C::K_PITCH + ((((QK8 ? 4 : 2) * s + KH * g + hh) ^ swz_row<C::K_PITCH>(r)) * 16);
+      k_rd[s][hh] = lds_base + C::K_ST0 + r * C::K_PITCH + ((((QK8 ? 4 : 2) * s + KH * g + hh) ^ swz_row<C::K_PITCH>(r)) * 16);
   // V operand: see the file comment.  li = lane within its block of 16.
   const int li = lane & 15;
-  int v_rd[DB];
-  int vt_rd[2] = {0, 0};
+  uint32_t v_rd[DB];
+  uint32_t vt_rd[2] = {0, 0};
   if constexpr (C::VT) {  // row d = 32db + r of the [d][key] tile, chunks 2g and 2g+1 = keys 32g .. 32g+31
 #pragma unroll
-    for (int hh = 0; hh < 2; ++hh) vt_rd[hh] = r * C::V_PITCH + (((2 * g + hh) ^ swz_row<C::V_PITCH>(r)) * 16);
+    for (int hh = 0; hh < 2; ++hh) vt_rd[hh] = lds_base + C::V_ST0 + r * C::V_PITCH + (((2 * g + hh) ^ swz_row<C::V_PITCH>(r)) * 16);
 #pragma unroll
     for (int db = 0; db < DB; ++db) v_rd[db] = 0;
   } else if constexpr (PV8) {
@@ -226,13 +239,13 @@ fmha_fwd_kernel(const FmhaArgs a) {
     const int v_key = 8 * (row_e >> 2) + 4 * g + (row_e & 3);  // + 16 u
 #pragma unroll
     for (int db = 0; db < DB; ++db)
-      v_rd[db] = v_key * C::V_PITCH + (((2 * db + ((lane >> 4) & 1)) ^ swz_v8<C::V_PITCH>(v_key)) * 16) + 8 * (li & 1);
+      v_rd[db] = lds_base + C::V_ST0 + v_key * C::V_PITCH + (((2 * db + ((lane >> 4) & 1)) ^ swz_v8<C::V_PITCH>(v_key)) * 16) + 8 * (li & 1);
   } else {
     const int v_key = 4 * g + (li >> 2);                       // + 16 ps + 8 h2
     const int v_col = 16 * ((lane >> 4) & 1) + 4 * (li & 3);   // + 32 db   (element index)
 #pragma unroll
     for (int db = 0; db < DB; ++db)
-      v_rd[db] = v_key * C::V_PITCH + ((((db * 32 + v_col) >> 3) ^ swz_v16<C::V_PITCH>(v_key)) * 16) + (v_col & 7) * 2;
+      v_rd[db] = lds_base + C::V_ST0 + v_key * C::V_PITCH + ((((db * 32 + v_col) >> 3) ^ swz_v16<C::V_PITCH>(v_key)) * 16) + (v_col & 7) * 2;
   }
 
   f32x16 oacc[DB];
@@ -240,7 +253,10 @@ fmha_fwd_kernel(const FmhaArgs a) {
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
-  float m_ref = -INFINITY, m_true = -INFINITY, l_run = 0.f;  // softmax reference point, true running max, running sum
+  // softmax reference point; this lane's running max of the raw scores (half of the query's keys); running sum;
+  // raw-score threshold (m_ref + kTau) / c above which the reference point moves
+  float m_ref = -INFINITY, m_lane = -INFINITY, l_run = 0.f, thr_raw = -INFINITY;
+  const float inv_c = 1.0f / c_log2;
   // e4m3 P: the row sum is taken on the MFMA pipe, which has cycles to spare there while the VALU does not.  One
   // 16x16x128 MFMA per 64 keys multiplies P^T (the same registers that feed the second GEMM) by a 0/1 matrix:
   // B lane (n = lane%16, block lane/16) is this kernel's lane (q = lane%32, g = lane/32), i.e. the 32 keys of query
@@ -248,17 +264,37 @@ fmha_fwd_kernel(const FmhaArgs a) {
   // hold the sum over BOTH key halves of query n + 16*(i%2) = lane%32: every lane ends up with the sum of its own
   // query, no exchange needed.  It sums P as rounded to e4m3, the weights the second GEMM really applies.
   constexpr bool MFMA_SUM = PV8 && D <= 128;  // head dim 256 has no registers to spare, and twice the MFMA work per key
+  constexpr bool DOT_SUM = !PV8;              // fp16 P: v_dot2_f32_f16 adds two rounded weights per instruction
   f32x4 l_acc = {0.f, 0.f, 0.f, 0.f};
-  int8v sum_a;
+  PReg sum_a;
   {
-    const int one4 = (((lane >> 4) & 1) == ((lane >> 2) & 1)) ? 0x38383838 : 0;  // e4m3 1.0 = 0x38
+    const bool on = ((lane >> 4) & 1) == ((lane >> 2) & 1);
 #pragma unroll
-    for (int t = 0; t < 8; ++t) sum_a[t] = one4;
+    for (int t = 0; t < 8; ++t) {
+      if constexpr (PV8) sum_a[t] = on ? 0x38383838 : 0;  // e4m3 1.0 = 0x38
+      else sum_a[t] = on ? (_Float16)1.0f : (_Float16)0.0f;
+    }
   }
 
   // S^T = K . Q^T for the K tile in LDS stage `stage`
-  auto qk = [&](int stage, f32x16 (&sacc)[KB]) {
-    const char *kt = smem + C::K_ST0 + stage * C::K_TILE;
+  constexpr int NPRE = C::KPRE;
+  QReg kpre[NPRE ? NPRE : 1];
+  auto read_kfrag = [&](uint32_t kt, int s, int kb) -> QReg {
+    if constexpr (QK8) {
+      const int4v lo = *LDS_AT(int4v, kt + k_rd[s][0] + kb * 32 * C::K_PITCH);
+      const int4v hi = *LDS_AT(int4v, kt + k_rd[s][1] + kb * 32 * C::K_PITCH);
+      return int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    } else {
+      return *LDS_AT(half8, kt + k_rd[s][0] + kb * 32 * C::K_PITCH);
+    }
+  };
+  // the first NPRE fragments (order: K-step major, 32-key block minor) of the K tile in slot `stage`
+  auto prefetch_k = [&](int stage) {
+#pragma unroll
+    for (int f = 0; f < NPRE; ++f) kpre[f] = read_kfrag(stage * C::K_TILE, f / KB, f % KB);
+  };
+  auto qk = [&](int stage, f32x16 (&sacc)[KB], bool use_pre = false) {
+    const uint32_t kt = stage * C::K_TILE;
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -267,13 +303,12 @@ fmha_fwd_kernel(const FmhaArgs a) {
     for (int s = 0; s < KS; ++s)
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
+        QReg ka;
+        if (use_pre && s * KB + kb < NPRE) ka = kpre[s * KB + kb];
+        else ka = read_kfrag(kt, s, kb);
         if constexpr (QK8) {
-          const int4v lo = *(const int4v *)(kt + k_rd[s][0] + kb * 32 * C::K_PITCH);
-          const int4v hi = *(const int4v *)(kt + k_rd[s][1] + kb * 32 * C::K_PITCH);
-          const int8v ka = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           sacc[kb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka, qreg[s], sacc[kb], 0, 0, 0, 0, 0, 0);
         } else {
-          const half8 ka = *(const half8 *)(kt + k_rd[s][0] + kb * 32 * C::K_PITCH);
           sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[s], sacc[kb], 0, 0, 0);
         }
       }
@@ -293,17 +328,20 @@ fmha_fwd_kernel(const FmhaArgs a) {
           *(f32x4 *)(srow + key0) = sv;
         }
     }
+    // The common case needs no exchange with the lane that holds the query's other keys: a lane only tests its own
+    // half against the threshold, and the (rare, wave-uniform) slow path completes the max.
     float mx = sacc[0][0];
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sacc[kb][v]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * c_log2;
-    m_true = fmaxf(m_true, mx);
-    if (__builtin_amdgcn_ballot_w64(mx > m_ref + kTau) != 0) {
-      const float m_new = fmaxf(m_ref, mx - kPBias);
+      for (int v = 0; v < 16; ++v) mx = __builtin_fmaxf(mx, sacc[kb][v]);
+    m_lane = __builtin_fmaxf(m_lane, mx);
+    if (__builtin_amdgcn_ballot_w64(mx > thr_raw) != 0) {
+      const float mfull = fmaxf(mx, __shfl_xor(mx, 32, 64)) * c_log2;
+      const float m_new = fmaxf(m_ref, mfull - kPBias);
       const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
       m_ref = m_new;
+      thr_raw = (m_ref + kTau) * inv_c;
       l_run *= alpha;
       if constexpr (MFMA_SUM) l_acc *= alpha;
 #pragma unroll
@@ -324,7 +362,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           p[t] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][4 * w + t], c_log2, -m_ref));
-          if constexpr (!MFMA_SUM) rs += p[t];
+          if constexpr (!MFMA_SUM && !DOT_SUM) rs += p[t];
         }
         if constexpr (PV8) {  // slot 16 kb + 4 w + t
           // the two converts overwrite both halves of the word: its old content is irrelevant, and handing in
@@ -336,42 +374,56 @@ fmha_fwd_kernel(const FmhaArgs a) {
           for (int t = 0; t < 4; ++t) pb[kb * 2 + w / 2][4 * (w % 2) + t] = (_Float16)p[t];
         }
       }
+    if constexpr (DOT_SUM) {  // sum of P as rounded to fp16 (the weights the second GEMM applies), fp32 accumulation
+      const half2v one2 = {(_Float16)1.0f, (_Float16)1.0f};
+      float rs2 = 0.f;
+#pragma unroll
+      for (int ps = 0; ps < PS; ++ps)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const half2v pp = {pb[ps][2 * t], pb[ps][2 * t + 1]};
+          if ((ps * 4 + t) & 1) rs2 = __builtin_amdgcn_fdot2(pp, one2, rs2, false);
+          else rs = __builtin_amdgcn_fdot2(pp, one2, rs, false);
+        }
+      rs += rs2;
+    }
     l_run += rs;
   };
   // O^T += V^T . P^T for the V tile in LDS stage `stage`
-  auto pv = [&](int stage, const PReg (&pb)[PS]) {
-    const char *vt = smem + C::V_ST0 + stage * C::V_TILE;
+  auto pv = [&](uint32_t vt /* byte offset of the V slot */, const PReg (&pb)[PS]) {
     if constexpr (MFMA_SUM) {
 #pragma unroll
-      for (int ps = 0; ps < PS; ++ps)
-        l_acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(sum_a, pb[ps], l_acc, 0, 0, 0, 0, 0, 0);
+      for (int ps = 0; ps < PS; ++ps) {
+        if constexpr (PV8) l_acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(sum_a, pb[ps], l_acc, 0, 0, 0, 0, 0, 0);
+        else l_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(sum_a, pb[ps], l_acc, 0, 0, 0);
+      }
     }
 #pragma unroll
     for (int ps = 0; ps < PS; ++ps)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         if constexpr (C::VT) {
-          const int4v lo = *(const int4v *)(vt + vt_rd[0] + db * 32 * C::V_PITCH);
-          const int4v hi = *(const int4v *)(vt + vt_rd[1] + db * 32 * C::V_PITCH);
+          const int4v lo = *LDS_AT(int4v, vt + vt_rd[0] + db * 32 * C::V_PITCH);
+          const int4v hi = *LDS_AT(int4v, vt + vt_rd[1] + db * 32 * C::V_PITCH);
           const int8v va = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb[ps], oacc[db], 0, 0, 0, 0, 0, 0);
         } else if constexpr (PV8) {
           int8v va;
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
-            const int2v x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(int2v, vt + v_rd[db] + (ps * 64 + u * 16) * C::V_PITCH));
+            const int2v x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(int2v, vt + v_rd[db] + (ps * 64 + u * 16) * C::V_PITCH));
             va[2 * u] = x[0];
             va[2 * u + 1] = x[1];
           }
           oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb[ps], oacc[db], 0, 0, 0, 0, 0, 0);
         } else {
-          const char *vp = vt + v_rd[db] + ps * 16 * C::V_PITCH;
+          const uint32_t vp = vt + v_rd[db] + ps * 16 * C::V_PITCH;
           union {
             struct { short4v lo, hi; } s;
             half8 h;
           } va;
-          va.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, vp));
-          va.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, vp + 8 * C::V_PITCH));
+          va.s.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(short4v, vp));
+          va.s.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_AT(short4v, vp + 8 * C::V_PITCH));
           oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va.h, pb[ps], oacc[db], 0, 0, 0);
         }
       }
@@ -389,94 +441,282 @@ fmha_fwd_kernel(const FmhaArgs a) {
     PReg pb[PS];
     if (HAS_NEXT) qk(P ^ 1, s_nxt);
     softmax_exp(s_cur, pb);
-    pv(P, pb);
+    pv(P * C::V_TILE, pb);
     if (HAS_NEXT) row_max_and_rescale(s_nxt, j + 1);
     wait_lds_dma();   // this wave's copies have landed ...
     __syncthreads();  // ... and so have everybody else's; all reads of the stages about to be refilled are done
   };
 
-  // ---- prologue: K_0, V_0, K_1 in flight; S_0 and its row max
-  f32x16 s_a[KB], s_b[KB];
-  load_k(0, 0);
-  load_v(0, 0);
-  load_k(n_tiles > 1 ? 1 : 0, 1);
-  wait_lds_dma();
-  __syncthreads();
-  qk(0, s_a);
-  row_max_and_rescale(s_a, 0);
-  __syncthreads();  // every wave is done with K stage 0 before step 0 overwrites it
+  // Two sub-tiles per barrier (SUB = 2): sub-tile s of K lives in K slot s % 4, sub-tile t of V in V slot t % 4.
+  // Step J covers sub-tiles 2J and 2J+1.  On entry s_a = S_{2J} is finished and folded into m_ref; K sub-tiles
+  // 2J+1, 2J+2 and V sub-tiles 2J, 2J+1 are in LDS.  The step refills the slots last read by step J-1: K sub-tiles
+  // 2J+3, 2J+4 at its start, V sub-tiles 2J+2, 2J+3 between its halves.  LAST: sub-tile 2J+1 is the final one.
+  auto step2 = [&](auto parity, auto last, int J, f32x16 (&s_a)[KB], f32x16 (&s_b)[KB]) {
+    constexpr int P = decltype(parity)::value;
+    constexpr bool LAST = decltype(last)::value;
+    const int t0 = 2 * J, t_max = n_tiles - 1;
+    load_k(t0 + 3 < t_max ? t0 + 3 : t_max, (2 * P + 3) % 4);
+    load_k(t0 + 4 < t_max ? t0 + 4 : t_max, (2 * P) % 4);
+    {
+      PReg pb[PS];
+      qk((2 * P + 1) % 4, s_b);
+      softmax_exp(s_a, pb);
+      pv(((2 * P) % 4) * C::V_TILE, pb);
+      row_max_and_rescale(s_b, t0 + 1);
+    }
+    load_v(t0 + 2 < t_max ? t0 + 2 : t_max, (2 * P + 2) % 4);
+    load_v(t0 + 3 < t_max ? t0 + 3 : t_max, (2 * P + 3) % 4);
+    {
+      PReg pb[PS];
+      if (!LAST) qk((2 * P + 2) % 4, s_a);
+      softmax_exp(s_b, pb);
+      pv(((2 * P + 1) % 4) * C::V_TILE, pb);
+      if (!LAST) row_max_and_rescale(s_a, t0 + 2);
+    }
+    wait_lds_dma();
+    __syncthreads();
+  };
+
+  // K fragment prefetch (KPRE): K tile t lives in K slot t % 4 and is fetched two steps ahead, so the tile of the NEXT
+  // step's S = K.Q^T is complete before this step's barrier and its first fragments are read into registers in front
+  // of the barrier: the MFMA pipe restarts right behind it instead of waiting for LDS while all waves read at once.
+  // The copies are issued after the step's K reads, off the restart path.
+  auto step_p = [&](auto jmod4, auto has_next, int j, f32x16 (&s_cur)[KB], f32x16 (&s_nxt)[KB]) {
+    constexpr int J4 = decltype(jmod4)::value;
+    constexpr int P = J4 & 1;
+    constexpr bool HAS_NEXT = decltype(has_next)::value;
+    PReg pb[PS];
+    if (HAS_NEXT) qk((J4 + 1) % 4, s_nxt, true);
+    load_k(j + 3 < n_tiles ? j + 3 : n_tiles - 1, (J4 + 3) % 4);
+    load_v(j + 1 < n_tiles ? j + 1 : n_tiles - 1, P ^ 1);
+    softmax_exp(s_cur, pb);
+    pv(P * C::V_TILE, pb);
+    if (HAS_NEXT) {
+      prefetch_k((J4 + 2) % 4);
+      row_max_and_rescale(s_nxt, j + 1);
+    }
+    wait_lds_dma();
+    __syncthreads();
+  };
 
   using std::integral_constant;
-  int j = 0;
-  for (; j + 2 < n_tiles; j += 2) {
-    step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
-    step(integral_constant<int, 1>{}, integral_constant<bool, true>{}, j + 1, s_b, s_a);
-  }
-  if (j + 2 == n_tiles) {  // two tiles left: j (even) with a successor, then the last one
-    step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
-    step(integral_constant<int, 1>{}, integral_constant<bool, false>{}, j + 1, s_b, s_a);
-  } else {                 // one tile left (even index)
-    step(integral_constant<int, 0>{}, integral_constant<bool, false>{}, j, s_a, s_b);
+  f32x16 s_a[KB], s_b[KB];
+  if constexpr (C::KPRE > 0) {
+    // ---- prologue: K_0, K_1, K_2, V_0 in flight; S_0, its row max, first fragments of K_1.  n_tiles % 4 == 0.
+    using T = integral_constant<bool, true>;
+    using F = integral_constant<bool, false>;
+    const int t_max = n_tiles - 1;
+    load_k(0, 0);
+    load_v(0, 0);
+    load_k(1, 1);
+    load_k(2 < t_max ? 2 : t_max, 2);
+    wait_lds_dma();
+    __syncthreads();
+    qk(0, s_a);
+    prefetch_k(1);
+    row_max_and_rescale(s_a, 0);
+    int j = 0;
+    for (; j + 4 < n_tiles; j += 4) {
+      step_p(integral_constant<int, 0>{}, T{}, j, s_a, s_b);
+      step_p(integral_constant<int, 1>{}, T{}, j + 1, s_b, s_a);
+      step_p(integral_constant<int, 2>{}, T{}, j + 2, s_a, s_b);
+      step_p(integral_constant<int, 3>{}, T{}, j + 3, s_b, s_a);
+    }
+    step_p(integral_constant<int, 0>{}, T{}, j, s_a, s_b);
+    step_p(integral_constant<int, 1>{}, T{}, j + 1, s_b, s_a);
+    step_p(integral_constant<int, 2>{}, T{}, j + 2, s_a, s_b);
+    step_p(integral_constant<int, 3>{}, F{}, j + 3, s_b, s_a);
+  } else if constexpr (C::SUB == 2) {
+    // ---- prologue: K_0, K_1, K_2, V_0, V_1 in flight; S_0 and its row max.  n_tiles is even and >= 2.
+    const int t_max = n_tiles - 1;
+    load_k(0, 0);
+    load_v(0, 0);
+    load_k(1, 1);
+    load_k(2 < t_max ? 2 : t_max, 2);
+    load_v(1, 1);
+    wait_lds_dma();
+    __syncthreads();
+    qk(0, s_a);
+    row_max_and_rescale(s_a, 0);
+    __syncthreads();  // every wave is done with K slot 0 before step 0 overwrites it
+    const int n_steps = n_tiles / 2;
+    int J = 0;
+    for (; J + 2 < n_steps; J += 2) {
+      step2(integral_constant<int, 0>{}, integral_constant<bool, false>{}, J, s_a, s_b);
+      step2(integral_constant<int, 1>{}, integral_constant<bool, false>{}, J + 1, s_a, s_b);
+    }
+    if (J + 2 == n_steps) {
+      step2(integral_constant<int, 0>{}, integral_constant<bool, false>{}, J, s_a, s_b);
+      step2(integral_constant<int, 1>{}, integral_constant<bool, true>{}, J + 1, s_a, s_b);
+    } else {
+      step2(integral_constant<int, 0>{}, integral_constant<bool, true>{}, J, s_a, s_b);
+    }
+  } else {
+    // ---- prologue: K_0, V_0, K_1 in flight; S_0 and its row max
+    load_k(0, 0);
+    load_v(0, 0);
+    load_k(n_tiles > 1 ? 1 : 0, 1);
+    wait_lds_dma();
+    __syncthreads();
+    qk(0, s_a);
+    row_max_and_rescale(s_a, 0);
+    __syncthreads();  // every wave is done with K stage 0 before step 0 overwrites it
+
+    int j = 0;
+    for (; j + 2 < n_tiles; j += 2) {
+      step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
+      step(integral_constant<int, 1>{}, integral_constant<bool, true>{}, j + 1, s_b, s_a);
+    }
+    if (j + 2 == n_tiles) {  // two tiles left: j (even) with a successor, then the last one
+      step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
+      step(integral_constant<int, 1>{}, integral_constant<bool, false>{}, j + 1, s_b, s_a);
+    } else {                 // one tile left (even index)
+      step(integral_constant<int, 0>{}, integral_constant<bool, false>{}, j, s_a, s_b);
+    }
   }
 
   // ---- epilogue: O = out_scale * O / l (online_softmax.h:59-85), fp16, [B,S,H,D]; a lane holds 4 consecutive d
   const float l_tot = MFMA_SUM ? l_acc[0] : l_run + __shfl_xor(l_run, 32, 64);
   const float inv = a.out_scale / l_tot;
   const int qrow = q0 + r;
-  _Float16 *orow = Op + (int64_t)qrow * ld;
+  // The accumulator layout gives a lane 4 consecutive d of ONE row: stored directly, a wave-wide store would touch
+  // 32 rows with 16 bytes each.  The wave's 32 x D tile goes through its own LDS region instead (all staged tiles
+  // are dead after the loop's last barrier) and leaves as whole rows, 16 bytes per lane.
+  {
+    char *ot = smem + wave * (32 * C::O_PITCH);
 #pragma unroll
-  for (int db = 0; db < DB; ++db)
+    for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      half4 o4;
+      for (int i = 0; i < 4; ++i) {
+        half4 o4;
 #pragma unroll
-      for (int t = 0; t < 4; ++t) o4[t] = (_Float16)(oacc[db][4 * i + t] * inv);
-      *(half4 *)(orow + db * 32 + 8 * i + 4 * g) = o4;
+        for (int t = 0; t < 4; ++t) o4[t] = (_Float16)(oacc[db][4 * i + t] * inv);
+        *(half4 *)(ot + r * C::O_PITCH + (db * 32 + 8 * i + 4 * g) * 2) = o4;
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    constexpr int LPR = D / 8;        // lanes per output row (16 bytes each)
+    constexpr int RPP = 64 / LPR;     // rows per wave-wide store
+    const int orow_l = lane / LPR, ochunk = lane % LPR;
+#pragma unroll
+    for (int pass = 0; pass < 32 / RPP; ++pass) {
+      const int row = pass * RPP + orow_l;
+      const int4v val = *(const int4v *)(ot + row * C::O_PITCH + ochunk * 16);
+      *(int4v *)(Op + (int64_t)(q0 + row) * ld + ochunk * 8) = val;
     }
-  if (g == 0) {
-    const int64_t si = ((int64_t)b * a.H + h) * a.Sq + qrow;
-    // taps are reported against the true row max, as the reference's miOut / sPrimeOut are (fmha_epilogue.h:7-46)
-    if (a.row_max) a.row_max[si] = m_true;
-    if (a.row_sum) a.row_sum[si] = l_tot * __builtin_amdgcn_exp2f(m_ref - m_true);
   }
+  if (a.row_max || a.row_sum) {
+    const float m_true = fmaxf(m_lane, __shfl_xor(m_lane, 32, 64)) * c_log2;
+    if (g == 0) {
+      const int64_t si = ((int64_t)b * a.H + h) * a.Sq + qrow;
+      // taps are reported against the true row max, as the reference's miOut / sPrimeOut are (fmha_epilogue.h:7-46)
+      if (a.row_max) a.row_max[si] = m_true;
+      if (a.row_sum) a.row_sum[si] = l_tot * __builtin_amdgcn_exp2f(m_ref - m_true);
+    }
+  }
+}
+
+// One-time set-up of an instantiation: raise its dynamic-LDS limit.  Thread-safe (first calls of one shape from several
+// host threads), and callable ahead of any launch (cfk_init) so that a first call under stream capture finds it done.
+template <class C>
+hipError_t prepare_fmha_cfg() {
+  static std::once_flag once;
+  static hipError_t status = hipSuccess;
+  std::call_once(once, [] {
+    status = hipFuncSetAttribute((const void *)fmha_fwd_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+  });
+  return status;
 }
 
 template <class C>
 hipError_t launch_fmha_cfg(const FmhaArgs &a, hipStream_t s) {
-  static bool attr_done = false;  // one attribute call per instantiation and process
-  auto kern = fmha_fwd_kernel<C>;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    attr_done = true;
-  }
+  const hipError_t e = prepare_fmha_cfg<C>();
+  if (e != hipSuccess) return e;
   const int grid = a.B * a.H * (a.Sq / C::BM);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(C::T), C::LDS_BYTES, s, a);
+  hipLaunchKernelGGL(fmha_fwd_kernel<C>, dim3(grid), dim3(C::T), C::LDS_BYTES, s, a);
   return hipGetLastError();
 }
 
 template <class C>
 void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
   p->block_m = C::BM;
-  p->block_n = C::BN;
+  p->block_n = C::BN * C::SUB;
   p->lds_bytes = C::LDS_BYTES;
   p->threads = C::T;
   p->grid = bh * (sq / C::BM);
 }
 
-// CFK_FMHA_TILE=small|large forces the 128-row or the 256-row workgroup tile where both exist (tuning aid; the
-// reference picks its tile with -DQBLKSIZE/-DKBLKSIZE at compile time, src/fmha-pipeline/shared_storage.h:4-15).
-// Otherwise the large tile is used where it measured faster (`prefer_large`: the fp16-P paths) when
-// seqlen_q % 256 == 0 and there are enough workgroups to fill 256 CUs twice.
-inline bool use_large_tile(int sq, int bh, bool prefer_large = true) {
-  static const int forced = [] {
+// ---- tile selection.  The reference fixes its tile at compile time (-DQBLKSIZE / -DKBLKSIZE,
+// src/fmha-pipeline/shared_storage.h:4-15, swept by compile_run_all_config.sh:3-6); here every shape is built and one is
+// picked per call.  CFK_FMHA_TILE=<query rows>x<keys> (e.g. 256x128), or small | large for the query rows alone, states
+// a wish; a wish no instantiation can serve for the given shape is ignored.
+struct TileWish {
+  int bm, bn;  // 0 = no wish
+};
+inline TileWish tile_wish() {
+  static const TileWish w = [] {
+    TileWish t{0, 0};
     const char *e = getenv("CFK_FMHA_TILE");
-    if (!e) return -1;
-    return e[0] == 's' ? 0 : e[0] == 'l' ? 1 : -1;
+    if (!e) return t;
+    if (e[0] == 's') t.bm = 128;
+    else if (e[0] == 'l') t.bm = 256;
+    else {
+      int bm = 0, bn = 0;
+      if (sscanf(e, "%dx%d", &bm, &bn) == 2) t = TileWish{bm, bn};
+    }
+    return t;
   }();
-  if (sq % 256 != 0 || forced == 0) return false;
-  if (forced == 1) return true;
-  return prefer_large && (long long)bh * (sq / 256) >= 512;
+  return w;
+}
+
+template <class... Cs>
+struct CfgList {};
+
+// the shapes an instantiation can run: whole query tiles, whole key steps (four key tiles per loop turn with the K
+// fragment prefetch, two with the two-tile step)
+template <class C>
+constexpr bool fits(int sq, int skv) {
+  return sq % C::BM == 0 && skv % (C::BN * (C::KPRE ? 4 : C::SUB)) == 0;
+}
+
+// Calls f with the first instantiation of the list that fits the shape and the wish.  Without a wish for the query
+// rows, tiles above 128 rows are only taken for `big` problems (enough workgroups to fill 256 CUs twice).
+template <class F, class... Cs>
+bool first_fit(CfgList<Cs...>, int sq, int skv, bool big, TileWish w, F &&f) {
+  bool done = false;
+  auto try_one = [&](auto c) {
+    using C = decltype(c);
+    if (done || !fits<C>(sq, skv)) return;
+    if (w.bm ? C::BM != w.bm : (C::BM > 128 && !big)) return;
+    if (w.bn && C::BN * C::SUB != w.bn) return;
+    f(c);
+    done = true;
+  };
+  (try_one(Cs{}), ...);
+  return done;
+}
+
+// wish first (over every instantiation), then the automatic order, then -- for shapes nothing fits -- the fallback,
+// whose tile the caller's divisibility check then names in its error
+template <class All, class Auto, class Fallback, class F>
+void select_tile(int sq, int skv, int bh, F &&f) {
+  const bool big = sq % 256 == 0 && (long long)bh * (sq / 256) >= 512;
+  const TileWish w = tile_wish();
+  if ((w.bm || w.bn) && first_fit(All{}, sq, skv, big, w, f)) return;
+  if (first_fit(Auto{}, sq, skv, big, TileWish{0, 0}, f)) return;
+  f(Fallback{});
+}
+
+template <class... Cs>
+hipError_t prepare_all(CfgList<Cs...>) {
+  hipError_t e = hipSuccess;
+  auto one = [&](auto c) {
+    const hipError_t r = prepare_fmha_cfg<decltype(c)>();
+    if (e == hipSuccess) e = r;
+  };
+  (one(Cs{}), ...);
+  return e;
 }
 
 }  // namespace cfk

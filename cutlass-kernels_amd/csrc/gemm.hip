@@ -20,6 +20,8 @@
 // that a lane ends up with 4 consecutive n of one row m: 8-byte row-major stores.
 #include <type_traits>
 
+#include <mutex>
+
 #include "fmha_common.h"
 
 namespace cfk {
@@ -265,26 +267,40 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
 }
 
 template <class T, bool NN>
-hipError_t launch(const GemmArgs &g, hipStream_t s) {
-  constexpr int WN = 2, BKB = 64, NS = 4;
-  static bool attr_done = false;
-  auto kern = gemm_kernel<T, NN, WN, BKB, NS>;
-  constexpr int LDS_BYTES = NS * 2 * BM * BKB;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    if (e != hipSuccess) return e;
-    attr_done = true;
+struct GemmLaunch {
+  static constexpr int WN = 2, BKB = 64, NS = 4;
+  static constexpr int LDS_BYTES = NS * 2 * BM * BKB;
+  static constexpr auto kern = gemm_kernel<T, NN, WN, BKB, NS>;
+  // one-time set-up, thread-safe and callable ahead of any launch
+  static hipError_t prepare() {
+    static std::once_flag once;
+    static hipError_t status = hipSuccess;
+    std::call_once(once, [] {
+      status = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    });
+    return status;
   }
-  hipLaunchKernelGGL(kern, dim3((g.M / BM) * (g.N / BN), g.batch), dim3(2 * WN * 64), LDS_BYTES, s, (const T *)g.A,
-                     (const T *)g.B, (const T *)g.C, (T *)g.D, g.M, g.N, g.K, g.alpha, g.beta);
-  return hipGetLastError();
-}
+  static hipError_t launch(const GemmArgs &g, hipStream_t s) {
+    const hipError_t e = prepare();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((g.M / BM) * (g.N / BN), g.batch), dim3(2 * WN * 64), LDS_BYTES, s, (const T *)g.A,
+                       (const T *)g.B, (const T *)g.C, (T *)g.D, g.M, g.N, g.K, g.alpha, g.beta);
+    return hipGetLastError();
+  }
+};
 
 }  // namespace
 
 hipError_t launch_gemm(const GemmArgs &g, hipStream_t s) {
-  if (g.f32) return g.layout == 0 ? launch<float, false>(g, s) : hipErrorNotSupported;
-  return g.layout == 0 ? launch<_Float16, false>(g, s) : launch<_Float16, true>(g, s);
+  if (g.f32) return g.layout == 0 ? GemmLaunch<float, false>::launch(g, s) : hipErrorNotSupported;
+  return g.layout == 0 ? GemmLaunch<_Float16, false>::launch(g, s) : GemmLaunch<_Float16, true>::launch(g, s);
+}
+
+hipError_t prepare_gemm() {
+  hipError_t e = GemmLaunch<float, false>::prepare();
+  if (e == hipSuccess) e = GemmLaunch<_Float16, false>::prepare();
+  if (e == hipSuccess) e = GemmLaunch<_Float16, true>::prepare();
+  return e;
 }
 
 }  // namespace cfk

@@ -56,7 +56,8 @@ typedef struct cfk_fmha_fwd_params {
   int32_t batch;     /* BATCH                                                                                 */
   int32_t heads;     /* NUMHEADS                                                                              */
   int32_t seqlen_q;  /* SEQLEN: multiple of 128                                                               */
-  int32_t seqlen_kv; /* KEYLEN: multiple of the key tile cfk_fmha_forward_plan reports (64; 32 for fp16 V at 256)   */
+  int32_t seqlen_kv; /* KEYLEN: multiple of 64 (32 for fp16 V at head_dim 256); cfk_fmha_forward_plan reports the
+                        key tile actually chosen                                                              */
   int32_t head_dim;  /* HEADDIM: 64, 128 or 256 (fmha_forward.cu:746-761)                                     */
   int32_t v_layout;  /* cfk_v_layout                                                                          */
   const void *q;     /* [B, S_q,  H, D] dtype, D contiguous (fmha_forward.cu:151-152)                         */
@@ -75,7 +76,12 @@ typedef struct cfk_fmha_fwd_params {
   float *dbg_row_max; /* optional tap, [B, H, S_q] fp32: running row max in the log2 domain (score*scale*log2e),
                          the reference's miOut under COPYOUTMI (fmha_epilogue.h:7-46); NULL = off              */
   float *dbg_row_sum; /* optional tap, [B, H, S_q] fp32: row sum of exp2(t - max), not its reciprocal, the
-                         reference's sPrimeOut (fmha_forward.cu:668-672); NULL = off                           */
+                         reference's sPrimeOut (fmha_forward.cu:668-672); NULL = off.  The sum is taken over the
+                         weights AS ROUNDED to the precision of P (fp16, or e4m3 for v_dtype = CFK_FP8_E4M3) -- the
+                         weights the second GEMM applies, so that rows of O are exactly normalised -- where the
+                         reference sums the fp32 values before the cast (online_softmax.h:173-206).  The rounding
+                         is unbiased: the two sums agree to ~1e-4 relative (fp16) / < 1 % (e4m3).  One exception:
+                         e4m3 with head_dim 256 sums the fp32 values, as the reference does                    */
 } cfk_fmha_fwd_params;
 
 /* FMHA forward: O = softmax(softmax_scale * Q K^T) V per (batch, head); no mask, no dropout.
@@ -120,6 +126,12 @@ typedef struct cfk_gemm_params {
   void *d;
 } cfk_gemm_params;
 int cfk_gemm(const cfk_gemm_params *p, void *stream);
+
+/* Optional: performs the one-time per-process set-up of every kernel (raising their dynamic-LDS limits) on the
+ * current device.  Launch calls do the same on first use of a kernel, thread-safely; calling this first keeps that
+ * set-up out of latency-critical first calls and out of stream captures.  No counterpart in the reference, whose
+ * entry sets the attribute on every call (include/utils/cuda_launch.hpp:7-20).  Needs a gfx950 device. */
+int cfk_init(void);
 
 /* Message for the calling thread's most recent non-zero return ("" if none). */
 const char *cfk_last_error(void);
