@@ -20,6 +20,7 @@ struct FmhaArgs {
   float out_scale;   // v_descale (1 for fp16)
   float s_scale;     // softmax_scale * q_descale * k_descale (scales the score tap)
   int32_t v_layout;  // 0 = [B,S,H,D], 1 = [B,D,H,S]
+  float tau;         // the softmax reference point moves when a tile's max exceeds it by more than this (log2 domain)
 };
 
 struct FmhaPlan {

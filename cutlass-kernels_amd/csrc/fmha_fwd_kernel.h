@@ -39,10 +39,11 @@
 //    register sets that swap roles every step (the loop is unrolled by two).
 //  * Deferred rescale: the reference rescales O and l by exp2(m_old - m_new) on every tile (online_softmax.h:
 //    144-165).  Any reference point m_ref works as long as exp2(t - m_ref) stays representable, so m_ref only moves
-//    -- and O, l are only rescaled -- when a tile max exceeds it by more than kTau = 8 (P <= 256 fits fp16 and
-//    e4m3).  With e4m3 P the reference point additionally sits 7 below the row max, so P spans (0, 2^8] instead of
-//    (0, 1] and probabilities down to 2^-17 of the row max stay out of e4m3's flush zone (the reference casts P in
-//    (0,1] directly, fmha_consumer.h:54); the bias cancels in O/l.
+//    -- and O, l are only rescaled -- when a tile max exceeds the maximum it was set from by more than a threshold
+//    chosen by the host so that P <= 2^8 (exact range for fp16 and e4m3).  With e4m3 P the reference point
+//    additionally sits 7 below the row max, so P spans (0, 2^8] instead of (0, 1] and probabilities down to 2^-17 of
+//    the row max stay out of e4m3's flush zone (the reference casts P in (0,1] directly, fmha_consumer.h:54); the
+//    bias cancels in O/l.
 //      - e4m3 V given pre-transposed [B,D,H,S] (the reference's offline transpose): the tile is [d][key]; the K
 //        tile is loaded row-permuted instead so that a lane's P slots are 32 contiguous keys and the V^T operand
 //        is two plain ds_read_b128 (the counterpart of the reference's FP8NOSHFL key permutation, done on K, in
@@ -137,7 +138,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
   constexpr int KH = QK8 ? 2 : 1;              // 16-byte LDS reads per K operand
   constexpr int DB = D / 32;                   // 32-row blocks of O^T
   constexpr int PS = PV8 ? BN / 64 : BN / 16;  // K-steps of O^T
-  constexpr float kTau = 8.0f;                 // deferred-rescale threshold (log2 domain)
+  const float kTau = a.tau;                    // deferred-rescale threshold above the running max (log2 domain)
   constexpr float kPBias = PV8 ? 7.0f : 0.0f;  // the reference point sits this far below the row max
   using QReg = std::conditional_t<QK8, int8v, half8>;
   using PReg = std::conditional_t<PV8, int8v, half8>;
@@ -254,7 +255,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
   // softmax reference point; this lane's running max of the raw scores (half of the query's keys); running sum;
-  // raw-score threshold (m_ref + kTau) / c above which the reference point moves
+  // raw-score threshold (m_ref + kPBias + kTau) / c above which the reference point moves
   float m_ref = -INFINITY, m_lane = -INFINITY, l_run = 0.f, thr_raw = -INFINITY;
   const float inv_c = 1.0f / c_log2;
   // e4m3 P: the row sum is taken on the MFMA pipe, which has cycles to spare there while the VALU does not.  One
@@ -341,7 +342,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
       const float m_new = fmaxf(m_ref, mfull - kPBias);
       const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
       m_ref = m_new;
-      thr_raw = (m_ref + kTau) * inv_c;
+      thr_raw = (m_ref + kPBias + kTau) * inv_c;
       l_run *= alpha;
       if constexpr (MFMA_SUM) l_acc *= alpha;
 #pragma unroll

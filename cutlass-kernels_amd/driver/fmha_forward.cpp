@@ -10,6 +10,9 @@
 //                            amax applies per-tensor amax/448 scales and passes the descales to the library
 //   --gemm2-fp8=true         with --prec-type=2: true = P and V in e4m3 too (the reference built with -DGEMM2FP8),
 //                            false = hybrid, Q,K e4m3 with fp16 P,V (the reference's default build, :446-450)
+//   --v-layout=bshd|bdhs     with --prec-type=2 --gemm2-fp8=true: bdhs hands V over pre-transposed, [B,D,H,S], the
+//                            reference's offline transpose for its GEMM2FP8 build (:514-532); bshd (default) leaves the
+//                            transform to the kernel
 //   --verify-all=false       also checks the score / row-max / row-sum taps (the reference's -DCOPYOUTMM0
 //                            -DCOPYOUTMI build: gemm-check-1, max-check, sum-check, :640-676)
 //   --dump-dir=<dir>         writes q.bin k.bin v.bin o.bin (+ meta.txt) for an external checker
@@ -46,7 +49,7 @@ struct Options {
   int batch = 4, dim = 2048, head = 64, seq = 4096, iterations = 20, streams = 1, prec = 2;
   bool gemm2_fp8 = true;
   bool ref_check = false, print_values = false, print_diffs = false, verify_all = false, help = false, selftest = false;
-  std::string fp8_scales = "unit", dump_dir;
+  std::string fp8_scales = "unit", dump_dir, v_layout = "bshd";
 };
 
 bool parse_bool(const char *v) { return !strcmp(v, "true") || !strcmp(v, "1"); }
@@ -73,6 +76,7 @@ bool parse(int argc, char **argv, Options &o) {
     else if (key == "verify-all") o.verify_all = parse_bool(val);
     else if (key == "gemm2-fp8") o.gemm2_fp8 = parse_bool(val);
     else if (key == "dump-dir") o.dump_dir = val;
+    else if (key == "v-layout") o.v_layout = val;
     else if (key == "selftest-e4m3") o.selftest = true;
     else return false;
   }
@@ -95,7 +99,8 @@ void print_usage() {
       "  --print-diffs=<bool>        If true, prints every element that fails the check.\n"
       "  --fp8-scales=unit|amax      fp8 quantisation: unit scales (reference behaviour) or per-tensor amax.\n"
       "  --gemm2-fp8=<bool>          fp8 only: P and V in e4m3 too (default true); false = fp16 P and V.\n"
-      "  --verify-all=<bool>         Also check the row-max / row-sum taps.\n"
+      "  --v-layout=bshd|bdhs        fp8 V layout: [B,S,H,D] (default) or pre-transposed [B,D,H,S].\n"
+      "  --verify-all=<bool>         Also check the score / row-max / row-sum taps.\n"
       "  --dump-dir=<dir>            Write q.bin k.bin v.bin o.bin meta.txt there.\n");
 }
 
@@ -240,6 +245,15 @@ int main(int argc, char **argv) {
   const int B = opt.batch, S = opt.seq, D = opt.head, H = opt.dim / opt.head;
   const bool fp8 = opt.prec == 2;
   const bool v_fp8 = fp8 && opt.gemm2_fp8;
+  if (opt.v_layout != "bshd" && opt.v_layout != "bdhs") {
+    printf("Unsupported V layout: %s\n", opt.v_layout.c_str());
+    return 1;
+  }
+  const bool v_bdhs = opt.v_layout == "bdhs";
+  if (v_bdhs && !v_fp8) {
+    printf("--v-layout=bdhs is a layout of e4m3 V (--prec-type=2 --gemm2-fp8=true)\n");
+    return 1;
+  }
   const float softmax_scale = 1.0f / std::sqrt((float)D);
 
   cfk_fmha_fwd_params plan_q{};
@@ -249,6 +263,7 @@ int main(int argc, char **argv) {
   plan_q.heads = H;
   plan_q.seqlen_q = plan_q.seqlen_kv = S;
   plan_q.head_dim = D;
+  plan_q.v_layout = v_bdhs ? CFK_V_BDHS : CFK_V_BSHD;
   plan_q.softmax_scale = softmax_scale;
   plan_q.q_descale = plan_q.k_descale = plan_q.v_descale = 1.f;
   int bm = 0, bn = 0;
@@ -310,7 +325,16 @@ int main(int argc, char **argv) {
   if (check_scores) HIP_CHECK(hipMalloc(&dsc, n_scores * 4));
   HIP_CHECK(hipMemcpy(dq, qb.data(), n * esz, hipMemcpyHostToDevice));
   HIP_CHECK(hipMemcpy(dk, kb.data(), n * esz, hipMemcpyHostToDevice));
-  HIP_CHECK(hipMemcpy(dv, vb.data(), n * vesz, hipMemcpyHostToDevice));
+  if (v_bdhs) {  // [B,S,H,D] -> [B,D,H,S], done offline as the reference does (:514-532)
+    std::vector<uint8_t> vt(n);
+    for (int b = 0; b < B; ++b)
+      for (int sq = 0; sq < S; ++sq)
+        for (int h = 0; h < H; ++h)
+          for (int d = 0; d < D; ++d) vt[(((size_t)b * D + d) * H + h) * S + sq] = vb[(((size_t)b * S + sq) * H + h) * D + d];
+    HIP_CHECK(hipMemcpy(dv, vt.data(), n, hipMemcpyHostToDevice));
+  } else {
+    HIP_CHECK(hipMemcpy(dv, vb.data(), n * vesz, hipMemcpyHostToDevice));
+  }
   {  // O is pre-filled with -1 (fmha_forward.cu:501-502)
     std::vector<_Float16> neg(n, (_Float16)-1.0f);
     HIP_CHECK(hipMemcpy(dout, neg.data(), n * 2, hipMemcpyHostToDevice));
@@ -321,7 +345,10 @@ int main(int argc, char **argv) {
   if (opt.streams > 1)
     for (auto &s : streams) HIP_CHECK(hipStreamCreate(&s));
   const int Lb = B / opt.streams;
-  auto launch_all = [&](int iters, bool taps) -> int {
+  void *dout_tap = nullptr;  // O of the score-tap launch (a debug build of the kernel): only gemm-check-1 uses that launch
+  if (check_scores) HIP_CHECK(hipMalloc(&dout_tap, n * 2));
+  // taps: 0 = none, 1 = row max / row sum (the kernel that was timed), 2 = scores as well (debug build, O discarded)
+  auto launch_all = [&](int iters, int taps) -> int {
     for (int it = 0; it < iters; ++it)
       for (int i = 0; i < opt.streams; ++i) {
         cfk_fmha_fwd_params p = plan_q;
@@ -329,12 +356,12 @@ int main(int argc, char **argv) {
         p.q = (const char *)dq + off * esz;
         p.k = (const char *)dk + off * esz;
         p.v = (const char *)dv + off * vesz;
-        p.o = (char *)dout + off * 2;
+        p.o = (taps == 2 ? (char *)dout_tap : (char *)dout) + off * 2;
         p.q_descale = descale[0];
         p.k_descale = descale[1];
         p.v_descale = descale[2];
-        if (taps) {
-          if (dsc) p.dbg_s = dsc + (size_t)i * Lb * H * S * S;
+        if (taps == 2) p.dbg_s = dsc + (size_t)i * Lb * H * S * S;
+        if (taps == 1) {
           p.dbg_row_max = dmi + (size_t)i * Lb * H * S;
           p.dbg_row_sum = dsp + (size_t)i * Lb * H * S;
         }
@@ -348,13 +375,13 @@ int main(int argc, char **argv) {
   };
 
   const double fmha_flops = 4.0 * B * H * (double)S * S * D / 1.0e9;  // :572-573
-  if (launch_all(10, false) != 0) return 2;                            // warm-up (:578-581)
+  if (launch_all(10, 0) != 0) return 2;                                // warm-up (:578-581)
   HIP_CHECK(hipDeviceSynchronize());
   hipEvent_t e0, e1;
   HIP_CHECK(hipEventCreate(&e0));
   HIP_CHECK(hipEventCreate(&e1));
   HIP_CHECK(hipEventRecord(e0, streams[0]));
-  if (launch_all(opt.iterations, false) != 0) return 2;
+  if (launch_all(opt.iterations, 0) != 0) return 2;
   if (opt.streams > 1) HIP_CHECK(hipDeviceSynchronize());
   HIP_CHECK(hipEventRecord(e1, streams[0]));
   HIP_CHECK(hipEventSynchronize(e1));
@@ -363,7 +390,9 @@ int main(int argc, char **argv) {
   const double t = ms_total / 1e3 / opt.iterations;
   printf("CUTE_FMHA:     [%6.1f]Gflop/s  (%6.4f)ms\n", fmha_flops / t, t * 1000);  // line format of :595-597
 
-  if (launch_all(1, true) != 0) return 2;  // one more launch with the taps on
+  // one more launch of the SAME kernel with the row taps on: O, row max and row sum checked below come from it
+  if (launch_all(1, 1) != 0) return 2;
+  if (check_scores && launch_all(1, 2) != 0) return 2;  // scores: separate launch of the debug build
   HIP_CHECK(hipDeviceSynchronize());
   std::vector<_Float16> ho(n);
   HIP_CHECK(hipMemcpy(ho.data(), dout, n * 2, hipMemcpyDeviceToHost));
@@ -433,10 +462,10 @@ int main(int argc, char **argv) {
     const bool ok = verify_tensor(got, ref, opt.print_values, opt.print_diffs, err_expected);
     printf("gemm-check-2: %s\n", ok ? "Passed" : "Failed");
     failed += !ok;
-    hipFree(fq); hipFree(fk); hipFree(fv); hipFree(fo); hipFree(rmax); hipFree(rinv); hipFree(rsc);
+    (void)hipFree(fq); (void)hipFree(fk); (void)hipFree(fv); (void)hipFree(fo); (void)hipFree(rmax); (void)hipFree(rinv); (void)hipFree(rsc);
   }
   for (auto &s : streams)
-    if (s) hipStreamDestroy(s);
-  hipFree(dq); hipFree(dk); hipFree(dv); hipFree(dout); hipFree(dmi); hipFree(dsp); hipFree(dsc);
+    if (s) (void)hipStreamDestroy(s);
+  (void)hipFree(dq); (void)hipFree(dk); (void)hipFree(dv); (void)hipFree(dout); (void)hipFree(dout_tap); (void)hipFree(dmi); (void)hipFree(dsp); (void)hipFree(dsc);
   return failed ? 3 : 0;
 }

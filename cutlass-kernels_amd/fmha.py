@@ -84,10 +84,17 @@ def lib():
         l.cfk_gemm_f16.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p] * 3 + [ctypes.c_int32, ctypes.c_void_p]
         l.cfk_gemm.restype = ctypes.c_int
         l.cfk_gemm.argtypes = [ctypes.POINTER(GemmParams), ctypes.c_void_p]
+        l.cfk_init.restype = ctypes.c_int
+        l.cfk_init.argtypes = []
         l.cfk_last_error.restype = ctypes.c_char_p
         l.cfk_version.restype = ctypes.c_char_p
         _lib = l
     return _lib
+
+
+def init() -> None:
+    """``cfk_init``: one-time set-up of every kernel on the current device (optional; launches do it on demand)."""
+    _check(lib().cfk_init())
 
 
 def last_error() -> str:

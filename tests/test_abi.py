@@ -17,7 +17,8 @@ def _declared_functions():
 
 def test_library_exports_every_declared_symbol():
     names = _declared_functions()
-    assert {"cfk_fmha_forward", "cfk_fmha_forward_plan", "cfk_gemm", "cfk_gemm_f16", "cfk_last_error", "cfk_version"} <= set(names)
+    assert {"cfk_fmha_forward", "cfk_fmha_forward_plan", "cfk_gemm", "cfk_gemm_f16", "cfk_init", "cfk_last_error",
+            "cfk_version"} <= set(names)
     lib = ctypes.CDLL(pkg.lib_path())
     for n in names:
         assert getattr(lib, n) is not None, n
@@ -86,6 +87,41 @@ def test_error_paths_mirror_reference_driver():
     assert lib.cfk_gemm(ctypes.byref(g), None) == -2
     g.k, g.batch = 64, 0
     assert lib.cfk_gemm(ctypes.byref(g), None) == -1
+    # the kernel addresses a 256-row operand tile with 32-bit byte offsets: 256 * K * element size < 4 GiB
+    g.batch, g.k = 1, 1 << 22                   # fp32: 256 * 4 Mi * 4 B = 4 GiB
+    assert lib.cfk_gemm(ctypes.byref(g), None) == -2 and "K too large" in pkg.last_error()
+    g.dtype, g.k = pkg.CFK_FP16, 1 << 23        # fp16: 256 * 8 Mi * 2 B = 4 GiB
+    assert lib.cfk_gemm(ctypes.byref(g), None) == -2 and "K too large" in pkg.last_error()
+    g.k, g.layout, g.n = 64, 1, 1 << 25         # NN: 64 * N * 2 B = 4 GiB
+    assert lib.cfk_gemm(ctypes.byref(g), None) == -2 and "N too large" in pkg.last_error()
+
+
+def test_plan_query_from_many_host_threads():
+    # the plan query touches no GPU and keeps its error message per thread
+    import threading
+    errors = []
+
+    def worker(i):
+        try:
+            for _ in range(200):
+                d = (64, 128, 256)[i % 3]
+                bm, bn, lds, thr = pkg.fmha_forward_plan(pkg.CFK_FP16 if i % 2 else pkg.CFK_FP8_E4M3, 2, 4, 1024, 1024, d)
+                assert 1024 % bm == 0 and 1024 % bn == 0
+                try:
+                    pkg.fmha_forward_plan(pkg.CFK_FP16, 1, 1, 512, 512, 96 + i)
+                except pkg.CfkError as e:
+                    assert f"Unsupported head dim: {96 + i}" in str(e)   # this thread's own message
+                else:
+                    raise AssertionError("head dim must be rejected")
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
 
 
 def test_python_binding_refuses_cpu_tensors():

@@ -65,7 +65,8 @@ def _load_dump(d):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("prec,head,extra", [(1, 64, []), (1, 128, ["--num-cuda-streams=2"]), (1, 256, []),
-                                             (2, 128, []), (2, 128, ["--fp8-scales=amax"]), (2, 64, []), (2, 256, []), (2, 128, ["--gemm2-fp8=false"])])
+                                             (2, 128, []), (2, 128, ["--fp8-scales=amax"]), (2, 64, []), (2, 256, []), (2, 128, ["--gemm2-fp8=false"]),
+                                             (2, 128, ["--v-layout=bdhs"]), (2, 64, ["--v-layout=bdhs", "--fp8-scales=amax"])])
 def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
     # fp8 needs the reference's own sequence length for its percentage criterion; fp16 passes at any length
     seq = 2048 if prec == 2 else 512
@@ -81,6 +82,37 @@ def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
     ref = oracle.attention_f32(q, k, v)["O"]
     assert max_abs(o, ref) <= (TOL_FP16 if p == 1 else TOL_FP8)
     assert oracle.verify_tensor(o, ref, ERRPCT_FP16 if p == 1 else ERRPCT_FP8)[0]
+
+
+def test_driver_rejects_bdhs_for_fp16_v():
+    r = _run("--prec-type=1", "--v-layout=bdhs", check=False)
+    assert r.returncode != 0 and "bdhs" in r.stdout
+    r = _run("--prec-type=2", "--v-layout=hdbs", check=False)
+    assert r.returncode != 0 and "Unsupported V layout" in r.stdout
+
+
+@pytest.mark.gpu
+def test_sweep_script_verify_all_on_a_reduced_problem():
+    # run_all_config.sh (the counterpart of compile_run_all_config.sh) in its verify-all mode: every precision mode x
+    # head size x tile shape that exists, each with gemm-check-1 / max-check / sum-check / gemm-check-2
+    script = os.path.join(ROOT, "cutlass-kernels_amd", "driver", "run_all_config.sh")
+    env = dict(os.environ, BATCH="1", SEQ="2048", DIM="512")
+    r = subprocess.run(["bash", script, "verify-all"], env=env, capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stdout[-4000:] + r.stderr[-2000:]
+    blocks = r.stdout.split("CONFIG ")[1:]
+    assert len(blocks) == 26, len(blocks)
+    seen = set()
+    for blk in blocks:
+        head_line = blk.splitlines()[0]
+        mode, head, tile = (x.split("=")[1] for x in head_line.replace(",", "").split())
+        bm, bn = tile.split("x")
+        assert f"QBLK = {bm}" in blk and f"KBLK = {bn}" in blk, blk          # the wished tile is the one that ran
+        for line in ("gemm-check-1: Passed", "max-check: Passed", "sum-check: Passed", "gemm-check-2: Passed"):
+            assert line in blk, (head_line, blk)
+        assert "Failed" not in blk
+        seen.add((mode, head, tile))
+    assert len(seen) == 26
+    assert {m for m, _, _ in seen} == {"fp16", "fp8", "fp8-bdhs", "hybrid"}
 
 
 GEMM_DRIVER = os.path.join(ROOT, "cutlass-kernels_amd", "driver", "gemm")

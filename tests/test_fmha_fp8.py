@@ -1,6 +1,7 @@
 """GPU parity of the fp8 e4m3 FMHA forward (through the C-ABI) against the CPU oracle run on the DEQUANTISED
 operands, as the reference's own check does (src/fmha-pipeline/fmha_forward.cu:613-631).  Gates: max-abs error
-<= 5e-2, and the reference's error-percentage criterion at its fp8 threshold (fmha_forward.cu:638-639)."""
+<= 5e-2 everywhere; the reference's error-percentage criterion at its fp8 threshold (fmha_forward.cu:638-639) from
+S >= 2048 on; below that, "no worse than the reference's device algorithm emulated on the same operands"."""
 import numpy as np
 import pytest
 
@@ -26,6 +27,24 @@ def _run(q, k, v, per_tensor=True, **kw):
     return o.float().cpu().numpy(), (qf, kf, vf)
 
 
+def _reference_algorithm_error(qf, kf, vf, ref, D):
+    """Error of the REFERENCE's device algorithm against the fp32 oracle on the same operands: tiled online softmax
+    with P in (0, 1] cast straight to e4m3 (fmha_consumer.h:54, online_softmax.h:87-207), emulated in numpy.
+    Returns (max-abs, error-%)."""
+    B, _, H, _ = qf.shape
+    emu = np.empty_like(ref)
+    for b in range(B):
+        for h in range(H):
+            emu[b, :, h], _, _ = oracle.online_softmax_tiled(qf[b, :, h], kf[b, :, h], vf[b, :, h], 64,
+                                                             oracle.LOG2E / np.sqrt(np.float32(D)), p_cast="e4m3")
+    return max_abs(emu, ref), oracle.verify_tensor(emu, ref, ERRPCT_FP8)[1]
+
+
+# the kernel may not be worse than the reference's own algorithm by more than this factor (plus a floor for
+# shapes where both errors are tiny)
+EMU_FACTOR, EMU_ABS_FLOOR, EMU_PCT_FLOOR = 1.25, 1e-3, 1e-3
+
+
 def _check_full(B, S, H, D, per_tensor=True, seqlen_kv=None):
     q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=seqlen_kv)
     got, (qf, kf, vf) = _run(q, k, v, per_tensor)
@@ -34,11 +53,18 @@ def _check_full(B, S, H, D, per_tensor=True, seqlen_kv=None):
     ok, pct = oracle.verify_tensor(got, ref, ERRPCT_FP8)
     print(f"fp8 B={B} S={S}/{seqlen_kv or S} H={H} D={D} per_tensor={per_tensor}: max-abs {err:.3e}, error% {pct:.2e}")
     assert err <= TOL_FP8, err
-    # The reference's percentage criterion is calibrated for its own problem size (S = 4096, where the e4m3
-    # rounding noise of P averages over thousands of keys): it is enforced from S >= 2048 on; the short shapes
-    # here are held to the max-abs gate and to the e4m3-P emulation test below.
     if S >= 2048 and (seqlen_kv or S) >= 2048:
+        # the reference's own gate at its fp8 threshold (fmha_forward.cu:638-639), calibrated for its problem size
+        # (S = 4096, where the e4m3 rounding noise of P averages over thousands of keys)
         assert ok, pct
+    else:
+        # Short sequences: with few keys the e4m3 rounding of P does not average out and the reference's device
+        # algorithm itself misses that gate.  The criterion that replaces it: the kernel is no worse than that
+        # algorithm, emulated on the same operands, in both of the reference's error measures.
+        emu_err, emu_pct = _reference_algorithm_error(qf, kf, vf, ref, D)
+        print(f"    reference algorithm (P cast to e4m3, emulated): max-abs {emu_err:.3e}, error% {emu_pct:.2e}")
+        assert err <= EMU_FACTOR * emu_err + EMU_ABS_FLOOR, (err, emu_err)
+        assert pct <= EMU_FACTOR * emu_pct + EMU_PCT_FLOOR, (pct, emu_pct)
     return got, ref
 
 
@@ -62,18 +88,20 @@ def test_rectangular_q_kv():
     _check_full(1, 512, 2, 128, seqlen_kv=128)
 
 
-def test_matches_tiled_emulation_with_e4m3_p():
-    # against the numpy emulation of the kernel-side algorithm with P rounded to e4m3 the kernel agrees far more
-    # closely than against the fp32 attention: what is left is P's bias (a power of two) and fp16 output rounding
+def test_not_worse_than_the_reference_algorithm_with_e4m3_p():
+    # One head in detail: the kernel against the fp32 oracle and against the numpy emulation of the reference's
+    # algorithm (P in (0, 1] cast straight to e4m3).  The kernel keeps P 2^7 higher (small weights stay out of
+    # e4m3's flush zone) and sums the rounded weights, so it differs from the emulation by about as much as either
+    # differs from the fp32 result -- what is asserted is that its error is not the larger one.
     B, S, H, D = 1, 256, 1, 128
     q, k, v = pkg.testbed.qkv(B, S, H, D)
     got, (qf, kf, vf) = _run(q, k, v)
     ref = oracle.attention_f32(qf, kf, vf)["O"]
     emu, _, _ = oracle.online_softmax_tiled(qf[0, :, 0], kf[0, :, 0], vf[0, :, 0], 64, oracle.LOG2E / np.sqrt(D),
                                             p_cast="e4m3")
-    e_ref, e_emu = max_abs(got[0, :, 0], ref[0, :, 0]), max_abs(got[0, :, 0], emu)
-    print(f"vs fp32 attention {e_ref:.3e}; vs e4m3-P emulation {e_emu:.3e}")
-    assert e_ref <= TOL_FP8 and e_emu <= TOL_FP8
+    e_ref, e_emu, emu_ref = max_abs(got[0, :, 0], ref[0, :, 0]), max_abs(got[0, :, 0], emu), max_abs(emu, ref[0, :, 0])
+    print(f"kernel vs fp32 attention {e_ref:.3e}; kernel vs e4m3-P emulation {e_emu:.3e}; emulation vs fp32 {emu_ref:.3e}")
+    assert e_ref <= TOL_FP8 and e_ref <= EMU_FACTOR * emu_ref + EMU_ABS_FLOOR
 
 
 def test_exact_arithmetic_pins_the_v_layout_transform():
@@ -145,6 +173,30 @@ def test_hybrid_mode_fp8_qk_fp16_pv(B, S, H, D):
     assert err <= TOL_FP16 and ok
 
 
+def test_hybrid_production_size_picks_the_256_row_tile():
+    # a problem large enough for the automatic choice of the 256-row tile (batch*heads*(S/256) >= 512)
+    import torch
+    from _util import ERRPCT_FP16, TOL_FP16
+    B, S, H, D = 4, 2048, 16, 128
+    f = pkg.fmha
+    assert f.fmha_forward_plan(f.CFK_FP8_E4M3, B, H, S, S, D, v_dtype=f.CFK_FP16)[0] == 256
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    (qc, qs, qf), (kc, ks, kf) = _quant(q), _quant(k)
+    v16 = v.astype(np.float16)
+    o = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(v16), q_descale=qs, k_descale=ks)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    vf = v16.astype(np.float32)
+    ref = oracle.attention_f32(qf, kf, vf, bh_pairs=subset_pairs(B, H))["O"]
+    oracle.attention_f32(qf, kf, vf, bh_pairs=[(b, h) for b in range(B) for h in range(H)], row_start=11, row_step=61,
+                         out=ref)
+    sel = ~np.isnan(ref)
+    err = max_abs(got[sel], ref[sel])
+    ok, pct = oracle.verify_tensor(got[sel], ref[sel], ERRPCT_FP16)
+    print(f"hybrid 256-row tile: checked {sel.sum()} elements, max-abs {err:.3e}, error% {pct:.2e}")
+    assert err <= TOL_FP16 and ok and not np.any(np.isnan(got))
+
+
 def test_hybrid_exact_arithmetic():
     rng = np.random.default_rng(12)
     for D in (64, 128, 256):
@@ -182,6 +234,10 @@ def test_pretransposed_v_layout(B, S, H, D):
     assert max_abs(got, o2.float().cpu().numpy()) <= 2e-3   # same P, same V, different summation order
     if S >= 2048:
         assert oracle.verify_tensor(got, ref, ERRPCT_FP8)[0]
+    else:
+        emu_err, emu_pct = _reference_algorithm_error(qf, kf, vf, ref, D)
+        assert err <= EMU_FACTOR * emu_err + EMU_ABS_FLOOR, (err, emu_err)
+        assert oracle.verify_tensor(got, ref, ERRPCT_FP8)[1] <= EMU_FACTOR * emu_pct + EMU_PCT_FLOOR
 
 
 def test_pretransposed_v_exact_arithmetic():

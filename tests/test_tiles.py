@@ -1,0 +1,60 @@
+"""Every tile shape the library builds, forced through CFK_FMHA_TILE -- the run-time counterpart of the reference's
+compile-time -DQBLKSIZE / -DKBLKSIZE sweep (src/fmha-pipeline/compile_run_all_config.sh:3-6) -- checked against the CPU
+oracle.  The wish is read once per process, so each tile runs in a fresh interpreter (tests/tile_case.py)."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+from _util import ERRPCT_FP16, ERRPCT_FP8, ROOT, TOL_FP16, TOL_FP8, pkg
+
+# tile wish -> cases (mode:B,S,H,D) that have an instantiation of exactly that tile
+CASES = {
+    "128x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f8:1,2048,2,64", "f8:1,2048,2,128", "f8:1,2048,1,256",
+               "hyb:1,512,2,64", "hyb:1,512,2,128"],
+    "256x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f8:1,2048,2,128", "hyb:1,512,2,128"],
+    "128x128": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,384,2,128", "f8:1,2048,2,64", "f8:1,2048,2,128",
+                "f8:1,2048,1,256", "hyb:1,512,2,64"],
+    "256x128": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128,384", "f8:1,2048,2,128", "hyb:1,512,2,128"],
+    "128x32": ["f16:1,256,2,256", "hyb:1,256,2,256"],
+}
+
+
+def test_tile_wish_is_honoured_by_the_plan_without_gpu():
+    # the plan query needs no GPU; a wish no instantiation serves is ignored
+    f = pkg.fmha
+    code = ("import sys; sys.path.insert(0, %r); import __graft_entry__ as e; p = e.load_package(); f = p.fmha; "
+            "print(f.fmha_forward_plan(f.CFK_FP16, 2, 4, 512, 512, 128)[:2], f.fmha_forward_plan(f.CFK_FP16, 2, 4, 512, 512, 256)[:2], "
+            "f.fmha_forward_plan(f.CFK_FP8_E4M3, 2, 4, 512, 512, 128)[:2], f.fmha_forward_plan(f.CFK_FP16, 2, 4, 384, 384, 128)[:2])" % ROOT)
+    def plans(wish):
+        env = dict(os.environ)
+        env.pop("CFK_FMHA_TILE", None)
+        if wish:
+            env["CFK_FMHA_TILE"] = wish
+        return subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout.strip()
+    assert plans(None) == "(128, 64) (128, 32) (128, 64) (128, 64)"           # small problems: 128-row tiles
+    assert plans("256x128") == "(256, 128) (128, 32) (256, 128) (128, 64)"     # no such tile at head dim 256; 384 % 256 != 0
+    assert plans("large") == "(256, 64) (128, 32) (256, 64) (128, 64)"
+    assert plans("128x128") == "(128, 128) (128, 32) (128, 128) (128, 128)"
+    assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:2] == (256, 64)   # big problem: automatic choice
+    assert f.fmha_forward_plan(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128)[:2] == (256, 128)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("wish", sorted(CASES))
+def test_forced_tiles_match_the_oracle(wish):
+    env = dict(os.environ, CFK_FMHA_TILE=wish, PYTHONPATH=os.path.join(ROOT, "tests") + os.pathsep + ROOT)
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "tile_case.py"), *CASES[wish]], env=env,
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout + r.stderr
+    rows = [json.loads(l.split(" ", 1)[1]) for l in r.stdout.splitlines() if l.startswith("TILECASE ")]
+    assert len(rows) == len(CASES[wish])
+    bm, bn = (int(x) for x in wish.split("x"))
+    for row in rows:
+        print(row)
+        assert (row["block_m"], row["block_n"]) == (bm, bn), row     # the wished tile really ran
+        fp8 = row["case"].startswith("f8")
+        assert not row["nan"] and row["max_abs"] <= (TOL_FP8 if fp8 else TOL_FP16), row
+        assert row["err_pct"] <= (ERRPCT_FP8 if fp8 else ERRPCT_FP16), row
