@@ -11,13 +11,14 @@
 // (:386-389); C and D are row-major here.  gfx950 has no tf32/xf32 MFMA: fp32 operands multiply in full fp32.
 //
 // Workgroup = 4 waves (one per SIMD) on a 256 x 256 macro tile; wave (wm, wn) of a 2 x 2 grid owns 128 x 128 of C as
-// 4 x 4 MFMA blocks, its 256 accumulator registers in the AGPR half of the register file.  K tiles are 32 deep and go
-// through a ring of four LDS stages (32 KB each: A 16 KB + B 16 KB): the copy of tile kt+3 is issued, one 1 KB piece
-// after every four MFMAs, while tile kt multiplies.  Measured on MI355X, M=N=K=8192: the spread-out copies are worth
-// +15 % when the operands are constant (1.50 PFLOP/s; copies issued back to back fill the memory pipeline's queue and
-// stall the wave, and with one wave per SIMD the MFMA pipe with it); with U(-1,1) operands the board is power-limited
-// and every variant lands at 1.10-1.16 PFLOP/s.  The MFMA computes the TRANSPOSED block (rows = n, columns = m) so
-// that a lane ends up with 4 consecutive n of one row m: 8-byte row-major stores.
+// 4 x 4 MFMA blocks, its 256 accumulator registers in the AGPR half of the register file.  K tiles are 128 bytes deep
+// (64 halves / 32 floats) and go global -> registers -> LDS: ordinary 16-byte loads a tile ahead, parked in one of two
+// 64 KB LDS stages by ds_write_b128 while the other stage multiplies, one barrier per tile.  (An earlier version copied
+// global -> LDS directly through a ring of four 32-deep stages: with one wave per SIMD an LDS-destination load holds
+// up the issuing wave and with it the MFMA pipe.)  The MFMA computes the TRANSPOSED block (rows = n, columns = m); the
+// epilogue stages each 32 x 128 row of blocks through LDS and stores whole rows, 16 bytes per lane.
+// Measured on MI355X, M=N=K=8192 fp16 (earlier version -> this one): 1.50 -> 1.64 PFLOP/s on constant operands,
+// 1.17 -> 1.19 PFLOP/s on U(-1,1) operands, where the board is power-limited.
 #include <type_traits>
 
 #include <mutex>
@@ -32,6 +33,7 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int int4v __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 256, BN = 256;
 
@@ -42,12 +44,10 @@ __device__ __forceinline__ int swz_k(int row) { return PITCH == 128 ? (row >> 1)
 // 512-byte rows read with ds_read_b64_tr_b16 (4 consecutive k x 64 contiguous bytes)
 __device__ __forceinline__ int swz512(int row) { return (row & 3) << 2; }
 
-// WN = waves along n (2 along m always): 2 -> 4 waves of 128 x 128, one per SIMD (the shipped shape; a third less
-// LDS traffic per MFMA than 4 -> 8 waves of 128 x 64, two per SIMD).
-// T = element type of A, B, C, D (_Float16 or float); BKB = bytes of a K-contiguous tile row (32 halves or 16
-// floats at 64), NS = LDS stages (copies run NS-1 tiles ahead of the multiply).  blockIdx.y = problem of a batch.
-template <class T, bool NN, int WN, int BKB, int NS>
-__global__ void __launch_bounds__(2 * WN * 64) __attribute__((amdgpu_waves_per_eu(WN / 2, WN / 2)))
+// T = element type of A, B, C, D (_Float16 or float); BKB = bytes of a K-contiguous tile row (64 halves or 32 floats at
+// 128).  blockIdx.y = problem of a batch.  4 waves of 128 x 128, one per SIMD.
+template <class T, bool NN, int BKB>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restrict__ Cin, T *__restrict__ D, int M, int N,
             int K, float alpha, float beta) {
   constexpr bool F32 = sizeof(T) == 4;
@@ -60,13 +60,13 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, g = lane >> 5;
-  constexpr int NWAVES = 2 * WN;
-  constexpr int NB = BN / WN / 32;     // 32-column blocks per wave
+  constexpr int WN = 2, NWAVES = 4;
+  constexpr int NB = 4;                // 32-column blocks per wave
   constexpr int PITCH = BKB;           // bytes per K-contiguous LDS row
   constexpr int A_TILE = BM * PITCH;   // TN: B tile likewise (n rows); NN: BK rows (k) of 512 B
   constexpr int STAGE = 2 * A_TILE;
-  constexpr int CPW = A_TILE / 1024 / NWAVES;  // 1 KB copies per wave and operand tile
-  constexpr int RPC = 1024 / PITCH;    // rows per copy
+  constexpr int CPW = A_TILE / 1024 / NWAVES;  // 16-byte pieces per lane and operand tile
+  constexpr int RPC = 1024 / PITCH;    // rows per wave-wide 1 KB piece
   constexpr int KS = PITCH / 32;       // K-steps per tile: 32 bytes of a row (one 16-byte fragment per lane half) each
   const int wm = wave / WN, wn = wave % WN;
 
@@ -84,7 +84,6 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   const int tn = in_grp / rows_in_group;
   const int m0 = tm * BM, n0 = tn * BN;
 
-  const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
   const int64_t batch = blockIdx.y;  // packed strides M*K, N*K, M*N (reference: gemm.cu:519-521)
   A += batch * M * K;
   B += batch * N * K;
@@ -93,8 +92,12 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   const char *Ap = (const char *)(A + (int64_t)m0 * K);
   const char *Bp = NN ? (const char *)(B + n0) : (const char *)(B + (int64_t)n0 * K);
 
-  // ---- global -> LDS copies, 16 B per lane, 1 KB per wave-wide copy
-  // A (and B in TN): 8 rows of 128 B per copy; 32 copies per tile, 4 per wave.
+  // ---- global -> register -> LDS staging, 16 B per lane and piece.  Piece i of wave w covers tile rows
+  // (i*NWAVES + w)*RPC .. +RPC; lane l owns LDS slot (row l / CPR, chunk position l % CPR) of the piece and fetches
+  // chunk position ^ swz(row) of that row: the XOR swizzle is applied on the global side, LDS writes are linear.
+  // The loads are ordinary loads into registers (compiler-tracked), issued a tile ahead of the ds_write that parks
+  // them in LDS: unlike LDS-destination loads they do not hold up the issuing wave, which with one wave per SIMD
+  // would hold up the MFMA pipe.
   uint32_t goff_a[CPW], goff_b[CPW];
 #pragma unroll
   for (int i = 0; i < CPW; ++i) {
@@ -103,19 +106,24 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
     goff_a[i] = (uint32_t)row * (uint32_t)(K * ES) + (uint32_t)((cp ^ swz_k<PITCH>(row)) * 16);
     if (!NN) {
       goff_b[i] = goff_a[i];
-    } else {  // B tile is BK rows (k) of 512 B (256 n): 2 rows per copy
+    } else {  // B tile is BK rows (k) of 512 B (256 n): 2 rows per piece
       const int krow = (i * NWAVES + wave) * 2 + (lane >> 5);
       const int cpb = lane & 31;
       goff_b[i] = (uint32_t)krow * (uint32_t)(N * 2) + (uint32_t)((cpb ^ swz512(krow)) * 16);
     }
   }
-  auto load_stage = [&](int kt, int stage) {
-    const char *ga = Ap + (size_t)kt * PITCH;
-    const char *gb = NN ? Bp + (size_t)kt * BK * (size_t)(N * 2) : Bp + (size_t)kt * PITCH;
-#pragma unroll
-    for (int i = 0; i < CPW; ++i) lds_dma16(ga + goff_a[i], lds_base + stage * STAGE + (i * NWAVES + wave) * 1024);
-#pragma unroll
-    for (int i = 0; i < CPW; ++i) lds_dma16(gb + goff_b[i], lds_base + stage * STAGE + A_TILE + (i * NWAVES + wave) * 1024);
+  const uint32_t st_off = wave * 1024 + lane * 16;  // + (piece * NWAVES) * 1024 (+ A_TILE for B) + stage * STAGE
+  int4v stg[2 * CPW];                               // the tile in flight: A pieces, then B pieces
+  auto tile_ptrs = [&](int kt, const char *&ga, const char *&gb) {
+    ga = Ap + (size_t)kt * PITCH;
+    gb = NN ? Bp + (size_t)kt * BK * (size_t)(N * 2) : Bp + (size_t)kt * PITCH;
+  };
+  auto load_piece = [&](const char *ga, const char *gb, int c) {
+    stg[c] = c < CPW ? *(const int4v *)(ga + goff_a[c]) : *(const int4v *)(gb + goff_b[c - CPW]);
+  };
+  auto store_piece = [&](int stage, int c) {
+    char *dst = smem + stage * STAGE + st_off + (c < CPW ? c * NWAVES * 1024 : A_TILE + (c - CPW) * NWAVES * 1024);
+    *(int4v *)dst = stg[c];
   };
 
   // ---- LDS read addresses.  K-step s: lane (r, g) needs bytes 32s + 16g .. +16 of its row (fp16: k = 16s + 8g .. +8;
@@ -169,108 +177,129 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) aop[mb] = *(const Frag *)(st + a_rd[s] + mb * 32 * PITCH);
   };
-  // One copy (index c of the 2*CPW a wave issues per tile: first the A ones, then the B ones) of the tile at
-  // ga / gb into stage `fill`
-  auto load_copy = [&](const char *ga, const char *gb, int fill, int c) {
-    if (c < CPW) lds_dma16(ga + goff_a[c], lds_base + fill * STAGE + (c * NWAVES + wave) * 1024);
-    else lds_dma16(gb + goff_b[c - CPW], lds_base + fill * STAGE + A_TILE + ((c - CPW) * NWAVES + wave) * 1024);
-  };
-  // The multiplies of one K-step, with the copies [c0, c1) of the tile being prefetched spread between them: the
-  // L1 takes a 1 KB copy apart into sixteen 64-byte accesses, so copies issued back to back fill the memory
-  // pipeline's queue and stall the wave (and with it the MFMA pipe) at the next one.
-  auto mma = [&](const Frag (&aop)[4], const Frag (&bop)[NB], const char *ga, const char *gb, int fill, int c0, int c1) {
+  // The multiplies of one row of blocks of a K-step (4 MFMAs, or 16 for fp32 operands)
+  auto mma_row = [&](const Frag (&aop)[4], const Frag (&bop)[NB], int mb) {
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
+    for (int nb = 0; nb < NB; ++nb) {  // transposed block: MFMA rows = n (B operand first), columns = m
+      if constexpr (F32) {
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {  // transposed block: MFMA rows = n (B operand first), columns = m
-        if constexpr (F32) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-            acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(bop[nb][e], aop[mb][e], acc[mb][nb], 0, 0, 0);
-        } else {
-          acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop[mb], acc[mb][nb], 0, 0, 0);
-        }
+        for (int e = 0; e < 4; ++e)
+          acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(bop[nb][e], aop[mb][e], acc[mb][nb], 0, 0, 0);
+      } else {
+        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop[mb], acc[mb][nb], 0, 0, 0);
       }
-#pragma unroll
-      for (int c = c0 + mb; c < c1; c += 4) load_copy(ga, gb, fill, c);
-      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // Copies per wave and tile, and how they spread over the K-steps of the tile that is multiplied meanwhile.  With
-  // two stages the tile being copied is needed right after this tile's barrier, so its copies go with the first KS-1
-  // steps; with more stages they go with all KS steps and the wait leaves the younger tiles in flight.
+  // Pipeline: two LDS stages and one tile in registers.  While tile kt multiplies out of stage kt % 2, the registers
+  // (tile kt+1, loaded a tile ago) are written to the other stage -- whose readers passed the barrier that opened
+  // this tile -- and refilled with tile kt+2.  Stores and loads are spread over the tile's K-steps, all before the
+  // tile's barrier.  One barrier per tile.
   constexpr int CPT = 2 * CPW;
-  constexpr int PER_STEP = NS == 2 ? (CPT + KS - 2) / (KS - 1) : CPT / KS;
-  constexpr int IN_FLIGHT = NS == 2 ? 0 : (NS - 3) * CPT + (KS - 1) * PER_STEP;
-  auto wait_tile = [&]() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT) : "memory"); };
+  constexpr int ST_STEPS = KS > 1 ? KS - 1 : 1;
+  constexpr int ST_PER = (CPT + ST_STEPS - 1) / ST_STEPS;     // pieces per K-step
+  const char *ga, *gb;
+  tile_ptrs(0, ga, gb);
 #pragma unroll
-  for (int t0 = 0; t0 < NS - 1; ++t0) load_stage(t0 < k_tiles ? t0 : k_tiles - 1, t0);
-  wait_lds_dma();
+  for (int c = 0; c < CPT; ++c) load_piece(ga, gb, c);
+#pragma unroll
+  for (int c = 0; c < CPT; ++c) store_piece(0, c);
+  tile_ptrs(k_tiles > 1 ? 1 : 0, ga, gb);
+#pragma unroll
+  for (int c = 0; c < CPT; ++c) load_piece(ga, gb, c);
   __syncthreads();
   Frag aop[2][4], bop[2][NB];  // two operand register sets: K-step s+1 is fetched while K-step s multiplies
   fetch(smem, 0, aop[0], bop[0]);
   int stage = 0;
   for (int kt = 0; kt < k_tiles; ++kt) {
-    // the stage the previous tile was read from (its last reads were issued before that tile's barrier) is refilled
-    // with tile kt+NS-1 (clamped at the end: a surplus copy rewrites a stage nobody reads any more)
-    const int fill = stage == 0 ? NS - 1 : stage - 1;
-    const int ld_t = kt + NS - 1 < k_tiles ? kt + NS - 1 : k_tiles - 1;
-    const char *ga = Ap + (size_t)ld_t * PITCH;
-    const char *gb = NN ? Bp + (size_t)ld_t * BK * (size_t)(N * 2) : Bp + (size_t)ld_t * PITCH;
     const char *st = smem + stage * STAGE;
-    const int nstage = stage + 1 == NS ? 0 : stage + 1;
+    const int nstage = stage ^ 1;
+    tile_ptrs(kt + 2 < k_tiles ? kt + 2 : k_tiles - 1, ga, gb);  // clamped at the end: a surplus tile is loaded and dropped
     // sched_barrier(0): the compiler's scheduler would otherwise sink each fetch down to its first use and expose
     // the LDS latency in front of every multiply
 #pragma unroll
-    for (int s2 = 0; s2 + 1 < KS; ++s2) {
-      fetch(st, s2 + 1, aop[(s2 + 1) & 1], bop[(s2 + 1) & 1]);
+    for (int s2 = 0; s2 < KS; ++s2) {
+      if (s2 + 1 < KS) {
+        fetch(st, s2 + 1, aop[(s2 + 1) & 1], bop[(s2 + 1) & 1]);
+      } else {
+        __syncthreads();  // tile kt+1 is in LDS for everybody; all reads of this tile's stage have completed
+        fetch(smem + nstage * STAGE, 0, aop[0], bop[0]);  // first K-step of the next tile, ahead of this tile's last multiplies
+      }
       __builtin_amdgcn_sched_barrier(0);
-      mma(aop[s2 & 1], bop[s2 & 1], ga, gb, fill, s2 * PER_STEP, (s2 + 1) * PER_STEP < CPT ? (s2 + 1) * PER_STEP : CPT);
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) {
+        mma_row(aop[s2 & 1], bop[s2 & 1], mb);
+        if (s2 < ST_STEPS) {  // this K-step's share of the staging traffic: park pieces of tile kt+1, refetch them for kt+2
+#pragma unroll
+          for (int c = s2 * ST_PER + mb; c < (s2 + 1) * ST_PER && c < CPT; c += 4) {
+            store_piece(nstage, c);
+            load_piece(ga, gb, c);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    wait_tile();
-    __syncthreads();  // the next tile has landed for everybody
-    // first K-step of the next tile is fetched before the last multiply of this one
-    fetch(smem + nstage * STAGE, 0, aop[0], bop[0]);
-    __builtin_amdgcn_sched_barrier(0);
-    mma(aop[(KS - 1) & 1], bop[(KS - 1) & 1], ga, gb, fill, NS == 2 ? CPT : (KS - 1) * PER_STEP, CPT);
     stage = nstage;
   }
-  wait_lds_dma();  // no copy may still be writing LDS when the workgroup retires
 
-  // ---- epilogue: D = alpha * acc + beta * C in fp32 (src/cutlass-gemm/gemm.cu:318-324); lane (m = r, g) holds
-  // n = 8i + 4g + j of each block: 4 consecutive elements of a row per access
-  using Out4 = std::conditional_t<F32, f32x4, half4>;
+  // ---- epilogue: D = alpha * acc + beta * C in fp32 (src/cutlass-gemm/gemm.cu:318-324).  Lane (m = r, g) holds
+  // n = 8i + 4g + j of each block: stored directly, a wave-wide store would touch 32 rows with 16 or 32 bytes each.
+  // Each 32 x 128 row of blocks goes through the wave's own LDS region (the stages are dead: every wave passed the last
+  // tile's barrier after its last stage reads and writes) as raw fp32 accumulators and leaves as whole rows, 16 bytes
+  // per lane; alpha, beta and the single rounding to T are applied on the way out.
+  constexpr int E_PITCH = 128 * 4 + 16;          // bytes per staged row of 128 floats, padded
+  constexpr int EPL = 16 / ES;                   // elements per lane and store (8 halves / 4 floats)
+  constexpr int LPR = 128 / EPL, RPP = 64 / LPR; // lanes per row, rows per wave-wide store
+  using OutV = std::conditional_t<F32, f32x4, half8>;
   const bool with_c = Cin != nullptr && beta != 0.f;
+  char *et = smem + wave * (32 * E_PITCH);
+  const int e_row = lane / LPR, e_col = (lane % LPR) * EPL;
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
-    const int64_t row_off = (int64_t)(m0 + wm * 128 + mb * 32 + r) * N + n0 + wn * NB * 32;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int64_t off = row_off + nb * 32 + 8 * i + 4 * g;
-        float v[4];
+        f32x4 v4;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) v[j] = alpha * acc[mb][nb][4 * i + j];
-        if (with_c) {
-          const Out4 c4 = *(const Out4 *)(Cin + off);
-#pragma unroll
-          for (int j = 0; j < 4; ++j) v[j] += beta * (float)c4[j];
-        }
-        Out4 o4;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) o4[j] = (T)v[j];
-        *(Out4 *)(D + off) = o4;
+        for (int j = 0; j < 4; ++j) v4[j] = acc[mb][nb][4 * i + j];
+        *(f32x4 *)(et + r * E_PITCH + (nb * 32 + 8 * i + 4 * g) * 4) = v4;
       }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int pass = 0; pass < 32 / RPP; ++pass) {
+      const int row = pass * RPP + e_row;
+      const int64_t off = (int64_t)(m0 + wm * 128 + mb * 32 + row) * N + n0 + wn * NB * 32 + e_col;
+      float v[EPL];
+#pragma unroll
+      for (int q = 0; q < EPL / 4; ++q) {
+        const f32x4 x = *(const f32x4 *)(et + row * E_PITCH + (e_col + 4 * q) * 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[4 * q + j] = alpha * x[j];
+      }
+      if (with_c) {
+        const OutV c = *(const OutV *)(Cin + off);
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) v[j] += beta * (float)c[j];
+      }
+      OutV o;
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) o[j] = (T)v[j];
+      *(OutV *)(D + off) = o;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();  // the region is rewritten by the next row of blocks
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
   }
 }
 
 template <class T, bool NN>
 struct GemmLaunch {
-  static constexpr int WN = 2, BKB = 64, NS = 4;
-  static constexpr int LDS_BYTES = NS * 2 * BM * BKB;
-  static constexpr auto kern = gemm_kernel<T, NN, WN, BKB, NS>;
+  static constexpr int BKB = 128;  // 64-deep K tiles for fp16, 32-deep for fp32
+  static constexpr int LDS_BYTES = 2 * 2 * BM * BKB;
+  static constexpr auto kern = gemm_kernel<T, NN, BKB>;
   // one-time set-up, thread-safe and callable ahead of any launch
   static hipError_t prepare() {
     static std::once_flag once;
@@ -283,7 +312,7 @@ struct GemmLaunch {
   static hipError_t launch(const GemmArgs &g, hipStream_t s) {
     const hipError_t e = prepare();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((g.M / BM) * (g.N / BN), g.batch), dim3(2 * WN * 64), LDS_BYTES, s, (const T *)g.A,
+    hipLaunchKernelGGL(kern, dim3((g.M / BM) * (g.N / BN), g.batch), dim3(256), LDS_BYTES, s, (const T *)g.A,
                        (const T *)g.B, (const T *)g.C, (T *)g.D, g.M, g.N, g.K, g.alpha, g.beta);
     return hipGetLastError();
   }
