@@ -18,6 +18,7 @@ using C128_256x64P = FmhaCfg<128, 64, 8, 2, false, false, false, false, 1, 4>;  
 using C128_128x128 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 2>;
 using C128_256x128 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 2>;
 using C256_128x32 = FmhaCfg<256, 32, 4, 1, false, false>;
+using C256_128x32P = FmhaCfg<256, 32, 4, 1, false, false, false, false, 1, 4>;  // key length a multiple of 128
 
 // builds that also write the score tap (debug): 128-row tile only
 using C64Tap = FmhaCfg<64, 64, 4, 2, false, false, false, true>;
@@ -26,7 +27,9 @@ using C256Tap = FmhaCfg<256, 32, 4, 1, false, false, false, true>;
 
 using All64 = CfgList<C64_128x64, C64_256x64, C64_128x128, C64_256x128>;
 using All128 = CfgList<C128_128x64, C128_256x64P, C128_256x64, C128_128x128, C128_256x128>;
-using All256 = CfgList<C256_128x32>;  // two 32-key tiles per barrier spill registers inside the loop: not built
+// head dim 256: 64-key tiles and two 32-key tiles per barrier both spill registers inside the loop (572 against 940
+// TFLOP/s on B=2 H=8 S=8192): not built
+using All256 = CfgList<C256_128x32P, C256_128x32>;
 
 template <class F>
 bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
@@ -41,7 +44,7 @@ bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
   switch (head_dim) {
     case 64: select_tile<All64, CfgList<C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
     case 128: select_tile<All128, CfgList<C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
-    case 256: select_tile<All256, CfgList<C256_128x32>, C256_128x32>(sq, skv, bh, f); return true;
+    case 256: select_tile<All256, All256, C256_128x32>(sq, skv, bh, f); return true;
     default: return false;
   }
 }
