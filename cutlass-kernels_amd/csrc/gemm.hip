@@ -12,13 +12,16 @@
 //
 // Workgroup = 4 waves (one per SIMD) on a 256 x 256 macro tile; wave (wm, wn) of a 2 x 2 grid owns 128 x 128 of C as
 // 4 x 4 MFMA blocks, its 256 accumulator registers in the AGPR half of the register file.  K tiles are 128 bytes deep
-// (64 halves / 32 floats) and go global -> registers -> LDS: ordinary 16-byte loads a tile ahead, parked in one of two
-// 64 KB LDS stages by ds_write_b128 while the other stage multiplies, one barrier per tile.  (An earlier version copied
-// global -> LDS directly through a ring of four 32-deep stages: with one wave per SIMD an LDS-destination load holds
-// up the issuing wave and with it the MFMA pipe.)  The MFMA computes the TRANSPOSED block (rows = n, columns = m); the
-// epilogue stages each 32 x 128 row of blocks through LDS and stores whole rows, 16 bytes per lane.
-// Measured on MI355X, M=N=K=8192 fp16 (earlier version -> this one): 1.50 -> 1.64 PFLOP/s on constant operands,
-// 1.17 -> 1.19 PFLOP/s on U(-1,1) operands, where the board is power-limited.
+// (64 halves / 32 floats) and go global -> registers -> LDS: 16-byte buffer loads a tile ahead (scalar resource +
+// 32-bit lane offset, no vector address arithmetic), parked in one of two 64 KB LDS stages by ds_write_b128 while the
+// other stage multiplies, one barrier per tile; every multiply is followed by at most one fragment read or one
+// store/load pair, see the pipeline comment in the kernel.  (Global -> LDS copy instructions instead of the register
+// path, through a ring of four 32-deep stages and spread the same way, measured 1.57 against 1.94 PFLOP/s on constant
+// operands: with one wave per SIMD an LDS-destination load holds up the issuing wave and with it the MFMA pipe.)
+// The MFMA computes the TRANSPOSED block (rows = n, columns = m); the epilogue stages each 32 x 128 row of blocks
+// through LDS and stores whole rows, 16 bytes per lane.
+// Measured on MI355X, M=N=K=8192 fp16: 2.04 PFLOP/s on constant operands, 1.27-1.33 PFLOP/s on U(-1,1) operands,
+// where the board is power-limited.
 #include <type_traits>
 
 #include <mutex>
@@ -34,6 +37,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef short short4v __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int int4v __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int BM = 256, BN = 256;
 
@@ -114,12 +118,19 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   }
   const uint32_t st_off = wave * 1024 + lane * 16;  // + (piece * NWAVES) * 1024 (+ A_TILE for B) + stage * STAGE
   int4v stg[2 * CPW];                               // the tile in flight: A pieces, then B pieces
-  auto tile_ptrs = [&](int kt, const char *&ga, const char *&gb) {
-    ga = Ap + (size_t)kt * PITCH;
-    gb = NN ? Bp + (size_t)kt * BK * (size_t)(N * 2) : Bp + (size_t)kt * PITCH;
+  // Buffer loads: a scalar resource per operand tile (rebuilt per tile by the scalar unit) plus the lane's 32-bit
+  // offset, so that a load costs no vector address arithmetic.
+  using Rsrc = __amdgpu_buffer_rsrc_t;
+  auto tile_ptrs = [&](int kt, Rsrc &ga, Rsrc &gb) {
+    const char *pa = Ap + (size_t)kt * PITCH;
+    const char *pb = NN ? Bp + (size_t)kt * BK * (size_t)(N * 2) : Bp + (size_t)kt * PITCH;
+    ga = __builtin_amdgcn_make_buffer_rsrc((void *)pa, 0, -1, 0x00020000);
+    gb = __builtin_amdgcn_make_buffer_rsrc((void *)pb, 0, -1, 0x00020000);
   };
-  auto load_piece = [&](const char *ga, const char *gb, int c) {
-    stg[c] = c < CPW ? *(const int4v *)(ga + goff_a[c]) : *(const int4v *)(gb + goff_b[c - CPW]);
+  auto load_piece = [&](Rsrc ga, Rsrc gb, int c) {
+    const u32x4 x = c < CPW ? __builtin_amdgcn_raw_buffer_load_b128(ga, (int)goff_a[c], 0, 0)
+                            : __builtin_amdgcn_raw_buffer_load_b128(gb, (int)goff_b[c - CPW], 0, 0);
+    stg[c] = __builtin_bit_cast(int4v, x);
   };
   auto store_piece = [&](int stage, int c) {
     char *dst = smem + stage * STAGE + st_off + (c < CPW ? c * NWAVES * 1024 : A_TILE + (c - CPW) * NWAVES * 1024);
@@ -155,50 +166,57 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
       for (int v = 0; v < 16; ++v) acc[mb][nb][v] = 0.f;
 
   const int k_tiles = K / BK;
-  // operand fetch for K-step s of the tile in LDS stage `st`
-  auto fetch = [&](const char *st, int s, Frag (&aop)[4], Frag (&bop)[NB]) {
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      if (!NN) {
-        bop[nb] = *(const Frag *)(st + b_rd[s] + nb * 32 * PITCH);
-      } else {
-        if constexpr (!F32) {
-          union {
-            struct { short4v lo, hi; } p;
-            half8 h;
-          } u;
-          const char *bp = st + bt_rd[nb] + s * 16 * 512;
-          u.p.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp));
-          u.p.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp + 4 * 512));
-          bop[nb] = u.h;
-        }
+  // One 16-byte operand fragment of K-step s of the tile in LDS stage `st`, in the order the multiplies first need
+  // them: i = 0: B block 0, 1: A block 0, 2..4: B blocks 1..3, 5..7: A blocks 1..3
+  auto fetch_one = [&](const char *st, int s, int i, Frag (&aop)[4], Frag (&bop)[NB]) {
+    const bool is_a = i == 1 || i >= 5;
+    const int blk = i == 0 ? 0 : i == 1 ? 0 : i <= 4 ? i - 1 : i - 4;
+    if (is_a) {
+      aop[blk] = *(const Frag *)(st + a_rd[s] + blk * 32 * PITCH);
+    } else if (!NN) {
+      bop[blk] = *(const Frag *)(st + b_rd[s] + blk * 32 * PITCH);
+    } else {
+      if constexpr (!F32) {
+        union {
+          struct { short4v lo, hi; } p;
+          half8 h;
+        } u;
+        const char *bp = st + bt_rd[blk] + s * 16 * 512;
+        u.p.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp));
+        u.p.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp + 4 * 512));
+        bop[blk] = u.h;
       }
     }
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb) aop[mb] = *(const Frag *)(st + a_rd[s] + mb * 32 * PITCH);
   };
-  // The multiplies of one row of blocks of a K-step (4 MFMAs, or 16 for fp32 operands)
-  auto mma_row = [&](const Frag (&aop)[4], const Frag (&bop)[NB], int mb) {
+  // One block multiply (one MFMA, or 4 for fp32 operands).  Transposed block: MFMA rows = n (B operand first)
+  auto mma_block = [&](const Frag (&aop)[4], const Frag (&bop)[NB], int mb, int nb) {
+    if constexpr (F32) {
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {  // transposed block: MFMA rows = n (B operand first), columns = m
-      if constexpr (F32) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-          acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(bop[nb][e], aop[mb][e], acc[mb][nb], 0, 0, 0);
-      } else {
-        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop[mb], acc[mb][nb], 0, 0, 0);
-      }
+      for (int e = 0; e < 4; ++e)
+        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(bop[nb][e], aop[mb][e], acc[mb][nb], 0, 0, 0);
+    } else {
+      acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop[mb], acc[mb][nb], 0, 0, 0);
     }
   };
 
   // Pipeline: two LDS stages and one tile in registers.  While tile kt multiplies out of stage kt % 2, the registers
   // (tile kt+1, loaded a tile ago) are written to the other stage -- whose readers passed the barrier that opened
-  // this tile -- and refilled with tile kt+2.  Stores and loads are spread over the tile's K-steps, all before the
-  // tile's barrier.  One barrier per tile.
+  // this tile -- and refilled with tile kt+2, all before the tile's one barrier.  With one wave per SIMD nothing but
+  // this wave's own instruction stream keeps the MFMA pipe fed: a run of LDS and memory instructions between two
+  // multiplies stalls it.  So every K-step is laid out as 16 slots of one block multiply plus at most a piece of the
+  // other work, pinned in that order: the even slots carry the eight fragment reads of the next K-step (or, behind
+  // the barrier, of the next tile's first); the odd slots of all K-steps but the last carry the staging, the
+  // ds_write of a piece of tile kt+1 and, LD_LAG odd slots later, the load of the same piece of tile kt+2 (a load
+  // issued right behind the store that frees its register waits for that store to have read it).
+  // Measured (8192^3, constant operands): 1.64 PFLOP/s with reads and staging in runs of 8 and 3 instructions, 1.94
+  // with one per slot, 2.04 with the lagged load.
   constexpr int CPT = 2 * CPW;
   constexpr int ST_STEPS = KS > 1 ? KS - 1 : 1;
   constexpr int ST_PER = (CPT + ST_STEPS - 1) / ST_STEPS;     // pieces per K-step
-  const char *ga, *gb;
+  constexpr int LD_LAG = 2;
+  static_assert(ST_PER + LD_LAG <= 8, "stores and lagged loads of a K-step must fit its eight odd slots");
+  auto st_slot = [](int c) { return (c / ST_PER) * 8 + c % ST_PER; };  // odd slot (of the tile) of piece c's store
+  Rsrc ga, gb;
   tile_ptrs(0, ga, gb);
 #pragma unroll
   for (int c = 0; c < CPT; ++c) load_piece(ga, gb, c);
@@ -209,32 +227,33 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   for (int c = 0; c < CPT; ++c) load_piece(ga, gb, c);
   __syncthreads();
   Frag aop[2][4], bop[2][NB];  // two operand register sets: K-step s+1 is fetched while K-step s multiplies
-  fetch(smem, 0, aop[0], bop[0]);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) fetch_one(smem, 0, i, aop[0], bop[0]);
   int stage = 0;
   for (int kt = 0; kt < k_tiles; ++kt) {
     const char *st = smem + stage * STAGE;
     const int nstage = stage ^ 1;
     tile_ptrs(kt + 2 < k_tiles ? kt + 2 : k_tiles - 1, ga, gb);  // clamped at the end: a surplus tile is loaded and dropped
-    // sched_barrier(0): the compiler's scheduler would otherwise sink each fetch down to its first use and expose
-    // the LDS latency in front of every multiply
 #pragma unroll
     for (int s2 = 0; s2 < KS; ++s2) {
-      if (s2 + 1 < KS) {
-        fetch(st, s2 + 1, aop[(s2 + 1) & 1], bop[(s2 + 1) & 1]);
-      } else {
-        __syncthreads();  // tile kt+1 is in LDS for everybody; all reads of this tile's stage have completed
-        fetch(smem + nstage * STAGE, 0, aop[0], bop[0]);  // first K-step of the next tile, ahead of this tile's last multiplies
-      }
-      __builtin_amdgcn_sched_barrier(0);
+      const bool last = s2 + 1 == KS;
+      // tile kt+1 is in LDS for everybody; all reads of this tile's stage have completed
+      if (last) __syncthreads();
+      const char *src = last ? smem + nstage * STAGE : st;
+      const int s_next = last ? 0 : s2 + 1;
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb) {
-        mma_row(aop[s2 & 1], bop[s2 & 1], mb);
-        if (s2 < ST_STEPS) {  // this K-step's share of the staging traffic: park pieces of tile kt+1, refetch them for kt+2
+      for (int i = 0; i < 16; ++i) {
+        mma_block(aop[s2 & 1], bop[s2 & 1], i / 4, i % 4);
+        if (i % 2 == 0) {
+          fetch_one(src, s_next, i / 2, aop[(s2 + 1) & 1], bop[(s2 + 1) & 1]);
+        } else {
+          const int t = s2 * 8 + i / 2;  // odd slot number within the tile
 #pragma unroll
-          for (int c = s2 * ST_PER + mb; c < (s2 + 1) * ST_PER && c < CPT; c += 4) {
-            store_piece(nstage, c);
-            load_piece(ga, gb, c);
-          }
+          for (int c = 0; c < CPT; ++c)
+            if (st_slot(c) == t) store_piece(nstage, c);
+#pragma unroll
+          for (int c = 0; c < CPT; ++c)
+            if (st_slot(c) + LD_LAG == t) load_piece(ga, gb, c);
         }
         __builtin_amdgcn_sched_barrier(0);
       }

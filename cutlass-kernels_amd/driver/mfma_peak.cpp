@@ -8,7 +8,9 @@
 // A second set of lines prices the other work of a real kernel in that regime: the same fp16 loop with v_fma_f32,
 // v_exp_f32 and 16-byte LDS reads (conflict-free, feeding the MFMA's A operand) added per MFMA.
 //
-//   mfma_peak [--ms=30] [--no-mix]     approximate run time per measurement; --no-mix skips the second set
+//   mfma_peak [--ms=30] [--no-mix] [--waves-per-simd=2]
+//       --ms: approximate run time per measurement; --no-mix skips the second set; --waves-per-simd=1|2: 4-wave
+//       workgroups per CU (the GEMM kernel runs one wave per SIMD, the attention kernels two)
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -162,12 +164,14 @@ static uint8_t e4m3_of(float x) {  // coarse encoder, good enough for operand st
 
 typedef void (*loop_kernel)(float *, int, long long *, const int *);
 
+static int g_waves_per_simd = 2;
+
 static int measure_kernel(loop_kernel kern, double flop_per_mfma, const char *label, const int *ddata, double target_ms, int cus) {
   float *dout;
   long long *dclk;
   HIP_CHECK(hipMalloc(&dout, 4));
   HIP_CHECK(hipMalloc(&dclk, 16));
-  const int grid = cus * 2;  // two 4-wave workgroups per CU = two waves per SIMD
+  const int grid = cus * g_waves_per_simd;  // 4-wave workgroups: one per CU and wave per SIMD
   int iters = 2000;
   hipEvent_t e0, e1;
   HIP_CHECK(hipEventCreate(&e0));
@@ -211,10 +215,12 @@ int main(int argc, char **argv) {
   for (int i = 1; i < argc; ++i) {
     if (!strncmp(argv[i], "--ms=", 5)) target_ms = atof(argv[i] + 5);
     if (!strcmp(argv[i], "--no-mix")) mix = false;
+    if (!strncmp(argv[i], "--waves-per-simd=", 17)) g_waves_per_simd = atoi(argv[i] + 17) == 1 ? 1 : 2;
   }
   hipDeviceProp_t prop;
   HIP_CHECK(hipGetDeviceProperties(&prop, 0));
-  printf("device: %s, %d CUs, nominal clock %.2f GHz\n", prop.gcnArchName, prop.multiProcessorCount, prop.clockRate / 1e6);
+  printf("device: %s, %d CUs, nominal clock %.2f GHz, %d wave(s) per SIMD\n", prop.gcnArchName, prop.multiProcessorCount, prop.clockRate / 1e6,
+         g_waves_per_simd);
   std::mt19937 gen(3081);
   std::normal_distribution<float> nd(0.f, 1.f);
   std::vector<int> h_const16(4096), h_rand16(4096), h_const8(4096), h_rand8(4096);
