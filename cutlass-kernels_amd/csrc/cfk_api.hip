@@ -103,6 +103,14 @@ int cfk_fmha_forward_plan(const cfk_fmha_fwd_params *params, int32_t *block_m, i
   return CFK_OK;
 }
 
+int cfk_fmha_forward_mfma(const cfk_fmha_fwd_params *params, int32_t *mfma_rows) {
+  cfk::FmhaPlan plan{};
+  int rc = check_fmha(params, &plan, false);
+  if (rc != CFK_OK) return rc;
+  if (mfma_rows) *mfma_rows = plan.mfma;
+  return CFK_OK;
+}
+
 int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
   cfk::FmhaPlan plan{};
   int rc = check_fmha(p, &plan, true);

@@ -25,6 +25,7 @@ struct FmhaArgs {
 
 struct FmhaPlan {
   int32_t block_m, block_n, lds_bytes, threads, grid;
+  int32_t mfma;  // 32: 32x32 MFMA build, 16: 16x16x32 build
 };
 
 // Each launcher validates nothing: the C-ABI layer has already checked shapes against the plan.

@@ -1,13 +1,15 @@
-// FMHA forward, fp16 operands: tile shapes and dispatch.  The kernel is in fmha_fwd_kernel.h.
-#include "fmha_fwd_kernel.h"
+// FMHA forward, fp16 operands: tile shapes and dispatch.  The kernels are in fmha_fwd_kernel.h (32x32 MFMAs) and
+// fmha_fwd_kernel16.h (16x16x32 MFMAs).
+#include "fmha_fwd_kernel16.h"
 
 namespace cfk {
 namespace {
 
 // <head dim, keys per tile, waves, waves per SIMD, e4m3 Q/K, e4m3 P/V, V transposed, score tap, tiles per barrier,
-//  K fragments read ahead of the barrier>.  4 waves = 128 query rows (two workgroups share a CU), 8 waves = 256 rows
-// (one workgroup per CU, half the K/V traffic per query row).  Two waves per SIMD, except head dim 64, whose 128-row
-// tile fits three (the faster choice there), and head dim 256 (Q + O fill half the register file: one).
+//  K fragments read ahead of the barrier, 16x16x32 build>.  4 waves = 128 query rows (two workgroups share a CU),
+// 8 waves = 256 rows (one workgroup per CU, half the K/V traffic per query row).  Two waves per SIMD, except head dim
+// 64, whose 128-row tile fits three (the faster choice there), and head dim 256 (Q + O fill half the register file:
+// one).
 using C64_128x64 = FmhaCfg<64, 64, 4, 3, false, false>;
 using C64_256x64 = FmhaCfg<64, 64, 8, 2, false, false>;
 using C64_128x128 = FmhaCfg<64, 64, 4, 2, false, false, false, false, 2>;
@@ -19,14 +21,20 @@ using C128_128x128 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 2>;
 using C128_256x128 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 2>;
 using C256_128x32 = FmhaCfg<256, 32, 4, 1, false, false>;
 using C256_128x32P = FmhaCfg<256, 32, 4, 1, false, false, false, false, 1, 4>;  // key length a multiple of 128
+// The builds on 16x16x32 MFMAs, the automatic choice for big problems at head dims 64 and 128 (+3..5 % on N(0,1)
+// data).  Not built: the K fragment prefetch and the two-tile step (registers spill or nothing is gained), 256 rows
+// at head dim 64 (880 against 919 TFLOP/s for 128 rows), head dim 256 (929 against 932 for the 32x32 build).
+using N64_128x64 = FmhaCfg<64, 64, 4, 3, false, false, false, false, 1, 0, true>;
+using N128_128x64 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 1, 0, true>;
+using N128_256x64 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 1, 0, true>;
 
 // builds that also write the score tap (debug): 128-row tile only
 using C64Tap = FmhaCfg<64, 64, 4, 2, false, false, false, true>;
 using C128Tap = FmhaCfg<128, 64, 4, 2, false, false, false, true>;
 using C256Tap = FmhaCfg<256, 32, 4, 1, false, false, false, true>;
 
-using All64 = CfgList<C64_128x64, C64_256x64, C64_128x128, C64_256x128>;
-using All128 = CfgList<C128_128x64, C128_256x64P, C128_256x64, C128_128x128, C128_256x128>;
+using All64 = CfgList<C64_128x64, N64_128x64, C64_256x64, C64_128x128, C64_256x128>;
+using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128>;
 // head dim 256: 64-key tiles and two 32-key tiles per barrier both spill registers inside the loop (572 against 940
 // TFLOP/s on B=2 H=8 S=8192): not built
 using All256 = CfgList<C256_128x32P, C256_128x32>;
@@ -42,8 +50,8 @@ bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
     }
   }
   switch (head_dim) {
-    case 64: select_tile<All64, CfgList<C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
-    case 128: select_tile<All128, CfgList<C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
+    case 64: select_tile<All64, CfgList<N64_128x64, C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
+    case 128: select_tile<All128, CfgList<N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
     case 256: select_tile<All256, All256, C256_128x32>(sq, skv, bh, f); return true;
     default: return false;
   }

@@ -69,9 +69,11 @@ typedef int int8v __attribute__((ext_vector_type(8)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int2v __attribute__((ext_vector_type(2)));
 
-template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_, bool VT_ = false, bool TAP_S_ = false, int SUB_ = 1, int KPRE_ = 0>
+template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_, bool VT_ = false, bool TAP_S_ = false, int SUB_ = 1, int KPRE_ = 0,
+          bool M16_ = false>
 struct FmhaCfg {
   static constexpr int D = D_, BN = BN_, NWAVES = NWAVES_;
+  static constexpr bool M16 = M16_;                             // the fp16 kernel on 16x16x32 MFMAs (fmha_fwd_kernel16.h)
   static constexpr int SUB = SUB_;                              // BN-key sub-tiles per barrier (1 or 2)
   static constexpr int KPRE = KPRE_;                            // K fragments of the next step read before the barrier
   static constexpr int NSLOT = KPRE ? 4 : 2 * SUB;              // LDS slots of one BN-key sub-tile of K
@@ -621,11 +623,21 @@ fmha_fwd_kernel(const FmhaArgs a) {
 // One-time set-up of an instantiation: raise its dynamic-LDS limit.  Thread-safe (first calls of one shape from several
 // host threads), and callable ahead of any launch (cfk_init) so that a first call under stream capture finds it done.
 template <class C>
+__global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(C::WPE, C::WPE))) fmha_fwd_kernel16(const FmhaArgs a);
+
+// the kernel an instantiation runs
+template <class C>
+constexpr auto fmha_kernel_of() {
+  if constexpr (C::M16) return &fmha_fwd_kernel16<C>;
+  else return &fmha_fwd_kernel<C>;
+}
+
+template <class C>
 hipError_t prepare_fmha_cfg() {
   static std::once_flag once;
   static hipError_t status = hipSuccess;
   std::call_once(once, [] {
-    status = hipFuncSetAttribute((const void *)fmha_fwd_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    status = hipFuncSetAttribute((const void *)fmha_kernel_of<C>(), hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
   });
   return status;
 }
@@ -635,7 +647,7 @@ hipError_t launch_fmha_cfg(const FmhaArgs &a, hipStream_t s) {
   const hipError_t e = prepare_fmha_cfg<C>();
   if (e != hipSuccess) return e;
   const int grid = a.B * a.H * (a.Sq / C::BM);
-  hipLaunchKernelGGL(fmha_fwd_kernel<C>, dim3(grid), dim3(C::T), C::LDS_BYTES, s, a);
+  hipLaunchKernelGGL(fmha_kernel_of<C>(), dim3(grid), dim3(C::T), C::LDS_BYTES, s, a);
   return hipGetLastError();
 }
 
@@ -643,6 +655,7 @@ template <class C>
 void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
   p->block_m = C::BM;
   p->block_n = C::BN * C::SUB;
+  p->mfma = C::M16 ? 16 : 32;
   p->lds_bytes = C::LDS_BYTES;
   p->threads = C::T;
   p->grid = bh * (sq / C::BM);
@@ -650,21 +663,24 @@ void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
 
 // ---- tile selection.  The reference fixes its tile at compile time (-DQBLKSIZE / -DKBLKSIZE,
 // src/fmha-pipeline/shared_storage.h:4-15, swept by compile_run_all_config.sh:3-6); here every shape is built and one is
-// picked per call.  CFK_FMHA_TILE=<query rows>x<keys> (e.g. 256x128), or small | large for the query rows alone, states
-// a wish; a wish no instantiation can serve for the given shape is ignored.
+// picked per call.  CFK_FMHA_TILE=<query rows>x<keys>[/16|/32] (e.g. 256x128, or 256x64/16 for the build on 16x16x32
+// MFMAs), or small | large for the query rows alone, states a wish; a wish no instantiation can serve for the given
+// shape is ignored.
 struct TileWish {
   int bm, bn;  // 0 = no wish
+  int mfma;    // 16 or 32: the MFMA shape of the build (fp16 kernels come in both); 0 = no wish
 };
 inline TileWish tile_wish() {
   static const TileWish w = [] {
-    TileWish t{0, 0};
+    TileWish t{0, 0, 0};
     const char *e = getenv("CFK_FMHA_TILE");
     if (!e) return t;
     if (e[0] == 's') t.bm = 128;
     else if (e[0] == 'l') t.bm = 256;
     else {
-      int bm = 0, bn = 0;
-      if (sscanf(e, "%dx%d", &bm, &bn) == 2) t = TileWish{bm, bn};
+      int bm = 0, bn = 0, mfma = 0;
+      const int n = sscanf(e, "%dx%d/%d", &bm, &bn, &mfma);
+      if (n >= 2) t = TileWish{bm, bn, n == 3 && (mfma == 16 || mfma == 32) ? mfma : 0};
     }
     return t;
   }();
@@ -682,15 +698,17 @@ constexpr bool fits(int sq, int skv) {
 }
 
 // Calls f with the first instantiation of the list that fits the shape and the wish.  Without a wish for the query
-// rows, tiles above 128 rows are only taken for `big` problems (enough workgroups to fill 256 CUs twice).
+// rows, tiles above 128 rows and the 16x16x32 builds (slower where launch and prologue dominate) are only taken for
+// `big` problems (enough workgroups to fill 256 CUs twice).
 template <class F, class... Cs>
 bool first_fit(CfgList<Cs...>, int sq, int skv, bool big, TileWish w, F &&f) {
   bool done = false;
   auto try_one = [&](auto c) {
     using C = decltype(c);
     if (done || !fits<C>(sq, skv)) return;
-    if (w.bm ? C::BM != w.bm : (C::BM > 128 && !big)) return;
+    if (w.bm ? C::BM != w.bm : ((C::BM > 128 || C::M16) && !big)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
+    if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;
     f(c);
     done = true;
   };
@@ -705,7 +723,7 @@ void select_tile(int sq, int skv, int bh, F &&f) {
   const bool big = sq % 256 == 0 && (long long)bh * (sq / 256) >= 512;
   const TileWish w = tile_wish();
   if ((w.bm || w.bn) && first_fit(All{}, sq, skv, big, w, f)) return;
-  if (first_fit(Auto{}, sq, skv, big, TileWish{0, 0}, f)) return;
+  if (first_fit(Auto{}, sq, skv, big, TileWish{0, 0, 0}, f)) return;
   f(Fallback{});
 }
 

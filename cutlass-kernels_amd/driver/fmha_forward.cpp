@@ -271,7 +271,9 @@ int main(int argc, char **argv) {
     printf("%s\n", cfk_last_error());
     return 1;
   }
-  printf("M = %d\nN = %d\nK = %d\nQBLK = %d\nKBLK = %d\nL = %d : %d * %d\n", S, S, D, bm, bn, H * B, H, B);
+  int mfma = 0;
+  cfk_fmha_forward_mfma(&plan_q, &mfma);
+  printf("M = %d\nN = %d\nK = %d\nQBLK = %d\nKBLK = %d\nMFMA = %dx%d\nL = %d : %d * %d\n", S, S, D, bm, bn, mfma, mfma, H * B, H, B);
 
   // seeded N(0,1) inputs, seeds 3080 + {1,2,3} (fmha_forward.cu:479-500)
   const size_t n = (size_t)B * S * H * D;

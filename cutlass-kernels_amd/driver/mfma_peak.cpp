@@ -63,7 +63,9 @@ __global__ void __launch_bounds__(256) mfma_loop(float *out, int iters, long lon
         half8 ha, hb;
         __builtin_memcpy(&ha, &a[u % 4], 16);
         __builtin_memcpy(&hb, &b[(u + 1) % 4], 16);
-        if (SMALL) c4[u % 8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ha, hb, c4[u % 8], 0, 0, 0);
+        // written out so that the accumulator is updated in place (through the builtin the register allocator
+        // rotates the eight small accumulators through copies, 56 moves per 16 multiplies)
+        if (SMALL) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c4[u % 8]) : "v"(ha), "v"(hb));
         else c[u % 4] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ha, hb, c[u % 4], 0, 0, 0);
       }
     }
@@ -215,7 +217,7 @@ int main(int argc, char **argv) {
   for (int i = 1; i < argc; ++i) {
     if (!strncmp(argv[i], "--ms=", 5)) target_ms = atof(argv[i] + 5);
     if (!strcmp(argv[i], "--no-mix")) mix = false;
-    if (!strncmp(argv[i], "--waves-per-simd=", 17)) g_waves_per_simd = atoi(argv[i] + 17) == 1 ? 1 : 2;
+    if (!strncmp(argv[i], "--waves-per-simd=", 17)) g_waves_per_simd = atoi(argv[i] + 17) < 1 ? 1 : atoi(argv[i] + 17) > 4 ? 4 : atoi(argv[i] + 17);
   }
   hipDeviceProp_t prop;
   HIP_CHECK(hipGetDeviceProperties(&prop, 0));

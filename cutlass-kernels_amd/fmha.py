@@ -80,6 +80,8 @@ def lib():
         l.cfk_fmha_forward.argtypes = [ctypes.POINTER(FmhaFwdParams), ctypes.c_void_p]
         l.cfk_fmha_forward_plan.restype = ctypes.c_int
         l.cfk_fmha_forward_plan.argtypes = [ctypes.POINTER(FmhaFwdParams)] + [ctypes.POINTER(ctypes.c_int32)] * 4
+        l.cfk_fmha_forward_mfma.restype = ctypes.c_int
+        l.cfk_fmha_forward_mfma.argtypes = [ctypes.POINTER(FmhaFwdParams), ctypes.POINTER(ctypes.c_int32)]
         l.cfk_gemm_f16.restype = ctypes.c_int
         l.cfk_gemm_f16.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p] * 3 + [ctypes.c_int32, ctypes.c_void_p]
         l.cfk_gemm.restype = ctypes.c_int
@@ -133,6 +135,14 @@ def fmha_forward_plan(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, v_layo
     out = [ctypes.c_int32() for _ in range(4)]
     _check(lib().cfk_fmha_forward_plan(ctypes.byref(p), *[ctypes.byref(x) for x in out]))
     return tuple(x.value for x in out)
+
+
+def fmha_forward_mfma(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, v_layout=CFK_V_BSHD, v_dtype=None):
+    """``cfk_fmha_forward_mfma``: 32 or 16, the MFMA shape of the kernel build the library picks.  No GPU needed."""
+    p = make_params(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, v_layout=v_layout, v_dtype=v_dtype)
+    out = ctypes.c_int32()
+    _check(lib().cfk_fmha_forward_mfma(ctypes.byref(p), ctypes.byref(out)))
+    return out.value
 
 
 def _stream_ptr(stream):

@@ -94,6 +94,13 @@ int cfk_fmha_forward(const cfk_fmha_fwd_params *params, void *stream);
 int cfk_fmha_forward_plan(const cfk_fmha_fwd_params *params, int32_t *block_m, int32_t *block_n,
                           int32_t *lds_bytes, int32_t *threads);
 
+/* The MFMA shape of the kernel build the library would pick for `params`: 32 (32x32x16 / 32x32x64 MFMAs) or 16
+ * (16x16x32; fp16 operands, big problems at head dims 64 and 128: the more power-efficient shape on this board).  No
+ * counterpart in the reference, whose MMA atom is fixed at compile time (src/fmha-pipeline/ss_helper.h:3-94).  The
+ * environment variable CFK_FMHA_TILE=<query rows>x<keys>[/16|/32] overrides the automatic choice of tile and shape.
+ * Does not touch the GPU. */
+int cfk_fmha_forward_mfma(const cfk_fmha_fwd_params *params, int32_t *mfma_rows);
+
 /* GEMM layouts for cfk_gemm_f16. */
 typedef enum cfk_gemm_layout {
   CFK_GEMM_TN = 0, /* A: M x K (K contiguous), B: N x K (K contiguous) -- the reference's form

@@ -19,6 +19,9 @@ CASES = {
                 "f8:1,2048,1,256", "hyb:1,512,2,64"],
     "256x128": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128,384", "f8:1,2048,2,128", "hyb:1,512,2,128"],
     "128x32": ["f16:1,256,2,256", "hyb:1,256,2,256"],
+    # the fp16 builds on 16x16x32 MFMAs
+    "128x64/16": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:2,384,3,128,192", "f16:1,256,2,64,64"],
+    "256x64/16": ["f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f16:2,256,1,128,64"],
 }
 
 
@@ -39,6 +42,13 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     assert plans("large") == "(256, 64) (128, 32) (256, 64) (128, 64)"
     assert plans("128x128") == "(128, 128) (128, 32) (128, 128) (128, 128)"
     assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:2] == (256, 64)   # big problem: automatic choice
+    # ... on 16x16x32 MFMAs for fp16 at head dims 64 and 128; small problems, head dim 256 and e4m3 stay on 32x32
+    assert f.fmha_forward_mfma(f.CFK_FP16, 8, 16, 2048, 2048, 128) == 16
+    assert f.fmha_forward_mfma(f.CFK_FP16, 4, 32, 4096, 4096, 64) == 16
+    assert f.fmha_forward_plan(f.CFK_FP16, 4, 32, 4096, 4096, 64)[:2] == (128, 64)
+    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 512, 512, 128) == 32
+    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 8, 8192, 8192, 256) == 32
+    assert f.fmha_forward_mfma(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128) == 32
     assert f.fmha_forward_plan(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128)[:2] == (256, 128)
 
 
@@ -51,10 +61,13 @@ def test_forced_tiles_match_the_oracle(wish):
     assert r.returncode == 0, r.stdout + r.stderr
     rows = [json.loads(l.split(" ", 1)[1]) for l in r.stdout.splitlines() if l.startswith("TILECASE ")]
     assert len(rows) == len(CASES[wish])
-    bm, bn = (int(x) for x in wish.split("x"))
+    shape, _, mfma = wish.partition("/")
+    bm, bn = (int(x) for x in shape.split("x"))
     for row in rows:
         print(row)
         assert (row["block_m"], row["block_n"]) == (bm, bn), row     # the wished tile really ran
+        if row["case"].startswith("f16"):
+            assert row["mfma"] == int(mfma or 32), row               # ... on the wished MFMA shape
         fp8 = row["case"].startswith("f8")
         assert not row["nan"] and row["max_abs"] <= (TOL_FP8 if fp8 else TOL_FP16), row
         assert row["err_pct"] <= (ERRPCT_FP8 if fp8 else ERRPCT_FP16), row

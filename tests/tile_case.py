@@ -21,9 +21,11 @@ def run_case(spec):
     Skv = vals[4] if len(vals) > 4 else S
     q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=Skv)
     f = pkg.fmha
+    mfma = 32
     if mode == "f16":
         q16, k16, v16 = (x.astype(np.float16) for x in (q, k, v))
         plan = f.fmha_forward_plan(f.CFK_FP16, B, H, S, Skv, D)
+        mfma = f.fmha_forward_mfma(f.CFK_FP16, B, H, S, Skv, D)
         o = pkg.fmha_forward(to_dev(q16), to_dev(k16), to_dev(v16))
         qf, kf, vf = (x.astype(np.float32) for x in (q16, k16, v16))
     else:
@@ -49,7 +51,7 @@ def run_case(spec):
                          out=ref)
     sel = ~np.isnan(ref)
     _, pct = oracle.verify_tensor(got[sel], ref[sel])
-    return dict(case=spec, block_m=plan[0], block_n=plan[1], lds_bytes=plan[2], checked=int(sel.sum()),
+    return dict(case=spec, block_m=plan[0], block_n=plan[1], mfma=mfma, lds_bytes=plan[2], checked=int(sel.sum()),
                 max_abs=max_abs(got[sel], ref[sel]), err_pct=pct, nan=bool(np.isnan(got).any()))
 
 
