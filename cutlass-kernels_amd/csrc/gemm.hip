@@ -10,18 +10,19 @@
 // read with ds_read_b64_tr_b16 exactly as V is in the attention kernel.  The reference writes C column-major
 // (:386-389); C and D are row-major here.  gfx950 has no tf32/xf32 MFMA: fp32 operands multiply in full fp32.
 //
-// Workgroup = 4 waves (one per SIMD) on a 256 x 256 macro tile; wave (wm, wn) of a 2 x 2 grid owns 128 x 128 of C as
-// 4 x 4 MFMA blocks, its 256 accumulator registers in the AGPR half of the register file.  K tiles are 128 bytes deep
-// (64 halves / 32 floats) and go global -> registers -> LDS: 16-byte buffer loads a tile ahead (scalar resource +
-// 32-bit lane offset, no vector address arithmetic), parked in one of two 64 KB LDS stages by ds_write_b128 while the
-// other stage multiplies, one barrier per tile; every multiply is followed by at most one fragment read or one
-// store/load pair, see the pipeline comment in the kernel.  (Global -> LDS copy instructions instead of the register
-// path, through a ring of four 32-deep stages and spread the same way, measured 1.57 against 1.94 PFLOP/s on constant
-// operands: with one wave per SIMD an LDS-destination load holds up the issuing wave and with it the MFMA pipe.)
-// The MFMA computes the TRANSPOSED block (rows = n, columns = m); the epilogue stages each 32 x 128 row of blocks
-// through LDS and stores whole rows, 16 bytes per lane.
-// Measured on MI355X, M=N=K=8192 fp16: 2.04 PFLOP/s on constant operands, 1.27-1.33 PFLOP/s on U(-1,1) operands,
-// where the board is power-limited.
+// Workgroup = 4 waves (one per SIMD) on a 256 x 256 macro tile; wave (wm, wn) of a 2 x 2 grid owns 128 x 128 of C, its
+// 256 accumulator registers in the AGPR half of the register file.  fp16 operands multiply on 16x16x32 MFMAs
+// (gemm_kernel16, 8 x 8 blocks per wave: the power-efficient shape on this board), fp32 operands on 32x32x2
+// (gemm_kernel, 4 x 4 blocks).  K tiles are 128 bytes deep (64 halves / 32 floats) and go global -> registers -> LDS:
+// 16-byte buffer loads a tile ahead (scalar resource + 32-bit lane offset, no vector address arithmetic), parked in
+// one of two 64 KB LDS stages by ds_write_b128 while the other stage multiplies, one barrier per tile; every multiply
+// is followed by at most one fragment read or one store/load pair, see the pipeline comments in the kernels.
+// (Global -> LDS copy instructions instead of the register path, through a ring of four 32-deep stages and spread the
+// same way, measured 1.57 against 1.94 PFLOP/s on constant operands: with one wave per SIMD an LDS-destination load
+// holds up the issuing wave and with it the MFMA pipe.)  The MFMA computes the TRANSPOSED block (rows = n, columns =
+// m); the epilogue stages each row of blocks through LDS and stores whole rows, 16 bytes per lane.
+// Measured on MI355X, M=N=K=8192 fp16 TN: 1.34-1.40 PFLOP/s on U(-1,1) operands, where the board is power-limited
+// (the vendor library's kernel for this shape, also on 16x16x32 MFMAs: 1.55); fp32: 152 TFLOP/s.
 #include <type_traits>
 
 #include <mutex>
@@ -314,11 +315,264 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   }
 }
 
+// 512-byte rows read with ds_read_b64_tr_b16 in the 16x16x32 lane map: a 32-lane half of the wave touches rows
+// 8g .. 8g+3 of two k groups g x 32 contiguous bytes; bit 0 stays clear so the 32 bytes stay contiguous
+__device__ __forceinline__ int swz512n(int row) { return ((row & 3) | (((row >> 3) & 1) << 2)) << 1; }
+
+// The fp16 kernel on 16x16x32 MFMAs (v_mfma_f32_16x16x32_f16): the same workgroup tile, staging path and epilogue as
+// gemm_kernel, with the wave's 128 x 128 of C as 8 x 8 blocks (NWAVES = 4; NWAVES = 8 runs two waves per SIMD on
+// 128 x 64 each and measured the same).  Measured, 8192^3 TN, same session: 1401 TFLOP/s on U(-1,1) operands against
+// 1309 for gemm_kernel<_Float16> (8 waves: 1390); on constant operands 1837 against 2048 (LDS writes between the
+// short multiplies hold the MFMA pipe up for about 20 cycles each).  On U(-1,1) operands this board is
+// power-limited and the deeper, narrower MFMA moves half the accumulator bits per FLOP: a register-only loop sustains
+// 1.90 PFLOP/s with it against 1.69 with 32x32x16.  Lane (c = lane % 16, g = lane / 16) holds, of an operand fragment,
+// row c and contraction slots 8g .. 8g+7 (16 bytes), and of an accumulator block column c, rows 4g .. 4g+3.  The MFMA
+// computes the transposed block (rows = n, columns = m), so a lane owns 4 consecutive n of one row m of C.
+template <bool NN, int NWAVES>
+__global__ void __launch_bounds__(NWAVES * 64) __attribute__((amdgpu_waves_per_eu(NWAVES / 4, NWAVES / 4)))
+gemm_kernel16(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, const _Float16 *__restrict__ Cin,
+              _Float16 *__restrict__ D, int M, int N, int K, float alpha, float beta) {
+  using T = _Float16;
+  constexpr int ES = 2, PITCH = 128, BK = PITCH / ES;  // 64-deep K tiles: two K-steps of 32
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c = lane & 15, g = lane >> 4;
+  constexpr int WN = NWAVES / 2;       // waves along n: the wave tile is 128 x 256/WN
+  constexpr int NB = 8;                // 16-row blocks per wave
+  constexpr int NBN = BN / WN / 16;    // 16-column blocks per wave
+  constexpr int A_TILE = BM * PITCH;   // TN: B tile likewise (n rows); NN: BK rows (k) of 512 B
+  constexpr int STAGE = 2 * A_TILE;
+  constexpr int CPW = A_TILE / 1024 / NWAVES;  // 16-byte pieces per lane and operand tile
+  constexpr int RPC = 1024 / PITCH;    // rows per wave-wide 1 KB piece
+  constexpr int KS = PITCH / 64;       // K-steps per tile: 64 bytes of a row (four 16-byte fragments, one per g) each
+  const int wm = wave / WN, wn = wave % WN;
+
+  // tile order and XCD remap as in gemm_kernel
+  const int tiles_n = N / BN, tiles_m = M / BM;
+  int t = xcd_remap(blockIdx.x, gridDim.x);
+  constexpr int GROUP = 8;
+  const int per_group = GROUP * tiles_n;
+  const int grp = t / per_group;
+  const int first_m = grp * GROUP;
+  const int rows_in_group = tiles_m - first_m < GROUP ? tiles_m - first_m : GROUP;
+  const int in_grp = t - grp * per_group;
+  const int tm = first_m + in_grp % rows_in_group;
+  const int tn = in_grp / rows_in_group;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int64_t batch = blockIdx.y;
+  A += batch * M * K;
+  B += batch * N * K;
+  D += batch * M * N;
+  if (Cin) Cin += batch * M * N;
+  const char *Ap = (const char *)(A + (int64_t)m0 * K);
+  const char *Bp = NN ? (const char *)(B + n0) : (const char *)(B + (int64_t)n0 * K);
+
+  // ---- global -> register -> LDS staging (see gemm_kernel)
+  uint32_t goff_a[CPW], goff_b[CPW];
+#pragma unroll
+  for (int i = 0; i < CPW; ++i) {
+    const int row = (i * NWAVES + wave) * RPC + lane / (PITCH / 16);
+    const int cp = lane % (PITCH / 16);
+    goff_a[i] = (uint32_t)row * (uint32_t)(K * ES) + (uint32_t)((cp ^ swz_k<PITCH>(row)) * 16);
+    if (!NN) {
+      goff_b[i] = goff_a[i];
+    } else {  // B tile is BK rows (k) of 512 B (256 n): 2 rows per piece
+      const int krow = (i * NWAVES + wave) * 2 + (lane >> 5);
+      const int cpb = lane & 31;
+      goff_b[i] = (uint32_t)krow * (uint32_t)(N * 2) + (uint32_t)((cpb ^ swz512n(krow)) * 16);
+    }
+  }
+  const uint32_t st_off = wave * 1024 + lane * 16;
+  int4v stg[2 * CPW];
+  using Rsrc = __amdgpu_buffer_rsrc_t;
+  auto tile_ptrs = [&](int kt, Rsrc &ga, Rsrc &gb) {
+    const char *pa = Ap + (size_t)kt * PITCH;
+    const char *pb = NN ? Bp + (size_t)kt * BK * (size_t)(N * 2) : Bp + (size_t)kt * PITCH;
+    ga = __builtin_amdgcn_make_buffer_rsrc((void *)pa, 0, -1, 0x00020000);
+    gb = __builtin_amdgcn_make_buffer_rsrc((void *)pb, 0, -1, 0x00020000);
+  };
+  auto load_piece = [&](Rsrc ga, Rsrc gb, int p) {
+    const u32x4 x = p < CPW ? __builtin_amdgcn_raw_buffer_load_b128(ga, (int)goff_a[p], 0, 0)
+                            : __builtin_amdgcn_raw_buffer_load_b128(gb, (int)goff_b[p - CPW], 0, 0);
+    stg[p] = __builtin_bit_cast(int4v, x);
+  };
+  auto store_piece = [&](int stage, int p) {
+    char *dst = smem + stage * STAGE + st_off + (p < CPW ? p * NWAVES * 1024 : A_TILE + (p - CPW) * NWAVES * 1024);
+    *(int4v *)dst = stg[p];
+  };
+
+  // ---- LDS read addresses.  K-step s: lane (c, g) needs bytes 64s + 16g .. +16 of its row (k = 32s + 8g .. +8).
+  // swz_k<128> depends on the row within its group of 16 only, so blocks are immediates.
+  int a_rd[KS], b_rd[KS];
+#pragma unroll
+  for (int s = 0; s < KS; ++s) {
+    a_rd[s] = (wm * 128 + c) * PITCH + (((4 * s + g) ^ swz_k<PITCH>(c)) * 16);                // + 16 rows per m block
+    b_rd[s] = A_TILE + (wn * NBN * 16 + c) * PITCH + (((4 * s + g) ^ swz_k<PITCH>(c)) * 16);       // + 16 rows per n block (TN)
+  }
+  // NN: the n-side operand via two ds_read_b64_tr_b16 from [k][n] rows: within its block of 16 lanes, lane L hands
+  // the read the address of (k row L/4, columns 4(L%4) .. +3) and receives k rows 0..3 of column L; block g reads k
+  // rows 8g .. 8g+3, the second read 4 further
+  const int bk_row = 8 * g + (c >> 2);          // + 32 s (+ 4)
+  const int cg = c & 3;
+  int bt_rd[NBN];
+#pragma unroll
+  for (int nb = 0; nb < NBN; ++nb) {
+    const int chunk = (wn * NBN * 16 + 16 * nb) / 8 + (cg >> 1);  // 16-byte chunk of the 512-byte row
+    bt_rd[nb] = A_TILE + bk_row * 512 + ((chunk ^ swz512n(bk_row)) * 16) + (cg & 1) * 8;
+  }
+
+  f32x4 acc[NB][NBN];  // [m block][n block]
+#pragma unroll
+  for (int mb = 0; mb < NB; ++mb)
+#pragma unroll
+    for (int nb = 0; nb < NBN; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int k_tiles = K / BK;
+  // operand fragments of K-step s of the tile in LDS stage `st`: m block blk, n block blk
+  auto fetch_a = [&](const char *st, int s, int blk) -> half8 { return *(const half8 *)(st + a_rd[s] + blk * 16 * PITCH); };
+  auto fetch_b = [&](const char *st, int s, int blk) -> half8 {
+    if constexpr (!NN) {
+      return *(const half8 *)(st + b_rd[s] + blk * 16 * PITCH);
+    } else {
+      union {
+        struct { short4v lo, hi; } p;
+        half8 h;
+      } u;
+      const char *bp = st + bt_rd[blk] + s * 32 * 512;
+      u.p.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp));
+      u.p.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp + 4 * 512));
+      return u.h;
+    }
+  };
+
+  // Pipeline as in gemm_kernel (two LDS stages, one tile in registers, one barrier per tile), laid out as slots of
+  // one multiply each (K-step major, then m block, then n block; SPM = NBN slots per m block) with at most one piece
+  // of other work behind each multiply, pinned in that order.  Fragment registers: the n-side fragments of a K-step
+  // are live throughout it and double-buffered (bop[K-step parity]); the m-side fragment of block mb is only needed
+  // for its NBN multiplies and lives in a ring of four (aop[mb % 4]), read two blocks ahead.
+  //   K-step 0:  first slot of m block mb: m fragment mb+2 (the last two: blocks 0, 1 of K-step 1);  slot SPM/2 of
+  //              m blocks 0 .. NBN-1: n fragment mb of K-step 1;  the CPT slots i % (NB*NBN/CPT) == 1: ds_write of a
+  //              staging piece of tile kt+1 and, LD_LAG pieces behind it, the load of the same piece of tile kt+2
+  //   K-step 1:  first slot of m blocks 0..5: m fragment mb+2;  first slot of m block 6: the barrier (every read of
+  //              this tile's stage and every write of the next tile's is in front of it), then one per slot the first
+  //              fragments of the next tile (n 0 .. NBN-1 and m 0, 1 of its K-step 0) in the order they are needed
+  constexpr int CPT = 2 * CPW;
+  constexpr int LD_LAG = 2;
+  constexpr int SPM = NBN;                    // slots per m block
+  constexpr int ST_EVERY = NB * NBN / CPT;    // a staging piece every so many slots of K-step 0
+  static_assert(KS == 2 && ST_EVERY >= 2 && NB * NBN % CPT == 0, "slot layout");
+  Rsrc ga, gb;
+  tile_ptrs(0, ga, gb);
+#pragma unroll
+  for (int p = 0; p < CPT; ++p) load_piece(ga, gb, p);
+#pragma unroll
+  for (int p = 0; p < CPT; ++p) store_piece(0, p);
+  tile_ptrs(k_tiles > 1 ? 1 : 0, ga, gb);
+#pragma unroll
+  for (int p = 0; p < CPT; ++p) load_piece(ga, gb, p);
+  __syncthreads();
+  half8 aop[4], bop[2][NBN];
+#pragma unroll
+  for (int nb = 0; nb < NBN; ++nb) bop[0][nb] = fetch_b(smem, 0, nb);
+  aop[0] = fetch_a(smem, 0, 0);
+  aop[1] = fetch_a(smem, 0, 1);
+  int stage = 0;
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    const char *st = smem + stage * STAGE;
+    const char *nx = smem + (stage ^ 1) * STAGE;
+    const int nstage = stage ^ 1;
+    tile_ptrs(kt + 2 < k_tiles ? kt + 2 : k_tiles - 1, ga, gb);  // clamped at the end: a surplus tile is loaded and dropped
+#pragma unroll
+    for (int s2 = 0; s2 < KS; ++s2) {
+#pragma unroll
+      for (int i = 0; i < NB * NBN; ++i) {
+        const int mb = i / SPM, nb = i % SPM;
+        if (s2 == 1 && i == 6 * SPM) __syncthreads();
+        // written out so that the accumulator is updated in place in the AGPR half: through the builtin the register
+        // allocator moves the small accumulators between the two halves (280 copies per tile).  Nothing but these
+        // multiplies touches the accumulators inside the loop, so no hazard is hidden from the compiler here.
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[mb][nb]) : "v"(bop[s2][nb]), "v"(aop[mb % 4]));
+        if (nb == 0 && (s2 == 0 || mb <= 5)) {
+          const int blk = mb + 2;
+          aop[blk % 4] = blk < NB ? fetch_a(st, s2, blk) : fetch_a(st, 1, blk - NB);
+        }
+        if (s2 == 0 && nb == SPM / 2 && mb < NBN) bop[1][mb] = fetch_b(st, 1, mb);
+        if (s2 == 1 && i >= 6 * SPM && i < 6 * SPM + NBN + 2) {
+          // n 0, m 0, n 1, m 1, n 2 ...
+          const int j = i - 6 * SPM;
+          if (j == 1) aop[0] = fetch_a(nx, 0, 0);
+          else if (j == 3) aop[1] = fetch_a(nx, 0, 1);
+          else bop[0][j == 0 ? 0 : j == 2 ? 1 : j - 2] = fetch_b(nx, 0, j == 0 ? 0 : j == 2 ? 1 : j - 2);
+        }
+        if (i % ST_EVERY == 1) {
+          const int q = (s2 * NB * NBN + i) / ST_EVERY;  // staging slot number within the tile
+          if (q < CPT) store_piece(nstage, q);
+          if (q >= LD_LAG && q - LD_LAG < CPT) load_piece(ga, gb, q - LD_LAG);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    stage = nstage;
+  }
+
+  // the last multiplies have left the pipe before the epilogue reads their accumulators (the compiler does not see
+  // the dependency through the asm statements)
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // ---- epilogue: D = alpha * acc + beta * C in fp32, each 16 x 128 row of blocks staged through the wave's own LDS
+  // region (see gemm_kernel) and stored as whole rows, 16 bytes per lane
+  constexpr int E_PITCH = 128 * 4 + 16;
+  constexpr int EPL = 8;                          // halves per lane and store
+  constexpr int WCOLS = NBN * 16;                   // columns of the wave tile
+  constexpr int LPR = WCOLS / EPL, RPP = 64 / LPR;  // lanes per row, rows per wave-wide store
+  const bool with_c = Cin != nullptr && beta != 0.f;
+  char *et = smem + wave * (16 * E_PITCH);
+  const int e_row = lane / LPR, e_col = (lane % LPR) * EPL;
+#pragma unroll
+  for (int mb = 0; mb < NB; ++mb) {
+#pragma unroll
+    for (int nb = 0; nb < NBN; ++nb) *(f32x4 *)(et + c * E_PITCH + (nb * 16 + 4 * g) * 4) = acc[mb][nb];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int pass = 0; pass < 16 / RPP; ++pass) {
+      const int row = pass * RPP + e_row;
+      const int64_t off = (int64_t)(m0 + wm * 128 + mb * 16 + row) * N + n0 + wn * WCOLS + e_col;
+      float v[EPL];
+#pragma unroll
+      for (int q = 0; q < EPL / 4; ++q) {
+        const f32x4 x = *(const f32x4 *)(et + row * E_PITCH + (e_col + 4 * q) * 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[4 * q + j] = alpha * x[j];
+      }
+      if (with_c) {
+        const half8 cv = *(const half8 *)(Cin + off);
+#pragma unroll
+        for (int j = 0; j < EPL; ++j) v[j] += beta * (float)cv[j];
+      }
+      half8 o;
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) o[j] = (T)v[j];
+      *(half8 *)(D + off) = o;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();  // the region is rewritten by the next row of blocks
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
+}
+
 template <class T, bool NN>
 struct GemmLaunch {
   static constexpr int BKB = 128;  // 64-deep K tiles for fp16, 32-deep for fp32
   static constexpr int LDS_BYTES = 2 * 2 * BM * BKB;
-  static constexpr auto kern = gemm_kernel<T, NN, BKB>;
+  static constexpr int WAVES16 = 4;  // waves of the fp16 kernel
+  static constexpr auto kern = [] {
+    if constexpr (sizeof(T) == 2) return gemm_kernel16<NN, WAVES16>;
+    else return gemm_kernel<T, NN, BKB>;
+  }();
   // one-time set-up, thread-safe and callable ahead of any launch
   static hipError_t prepare() {
     static std::once_flag once;
@@ -331,7 +585,7 @@ struct GemmLaunch {
   static hipError_t launch(const GemmArgs &g, hipStream_t s) {
     const hipError_t e = prepare();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((g.M / BM) * (g.N / BN), g.batch), dim3(256), LDS_BYTES, s, (const T *)g.A,
+    hipLaunchKernelGGL(kern, dim3((g.M / BM) * (g.N / BN), g.batch), dim3(sizeof(T) == 2 ? WAVES16 * 64 : 256), LDS_BYTES, s, (const T *)g.A,
                        (const T *)g.B, (const T *)g.C, (T *)g.D, g.M, g.N, g.K, g.alpha, g.beta);
     return hipGetLastError();
   }
