@@ -1,7 +1,7 @@
 // Dense (batched) GEMM D = alpha * A.B + beta * C with fp32 accumulation and an fp32 epilogue, D row-major M x N, for
-// fp16 operands (v_mfma_f32_32x32x16_f16) and fp32 operands (v_mfma_f32_32x32x2_f32) -- gfx950 only.
+// fp16 operands (v_mfma_f32_16x16x32_f16) and fp32 operands (v_mfma_f32_32x32x2_f32) -- gfx950 only.
 //
-// Secondary bench on the FMHA tile engine: the same LDS-DMA staging with XOR-swizzled rows and 32x32 MFMA tiles.
+// Secondary bench beside the attention kernels, with their XOR-swizzled LDS rows and transpose reads.
 // Takes the place of gemm_device/gemm of the reference's CuTe example (src/cute-gemm-tma-gma/gemm.cu:57-463: TMA load
 // of one A and one B tile, one synchronous WGMMA batch per K-tile, no pipelining; its type 1 is float, type 3 half,
 // :677-684; batch count L with packed strides, :519-521) and of the CUTLASS-API example with its alpha / beta
@@ -13,7 +13,7 @@
 // Workgroup = 4 waves (one per SIMD) on a 256 x 256 macro tile; wave (wm, wn) of a 2 x 2 grid owns 128 x 128 of C, its
 // 256 accumulator registers in the AGPR half of the register file.  fp16 operands multiply on 16x16x32 MFMAs
 // (gemm_kernel16, 8 x 8 blocks per wave: the power-efficient shape on this board), fp32 operands on 32x32x2
-// (gemm_kernel, 4 x 4 blocks).  K tiles are 128 bytes deep (64 halves / 32 floats) and go global -> registers -> LDS:
+// (gemm_kernel_f32, 4 x 4 blocks).  K tiles are 128 bytes deep (64 halves / 32 floats) and go global -> registers -> LDS:
 // 16-byte buffer loads a tile ahead (scalar resource + 32-bit lane offset, no vector address arithmetic), parked in
 // one of two 64 KB LDS stages by ds_write_b128 while the other stage multiplies, one barrier per tile; every multiply
 // is followed by at most one fragment read or one store/load pair, see the pipeline comments in the kernels.
@@ -46,20 +46,17 @@ constexpr int BM = 256, BN = 256;
 // 16-byte chunk index must spread over all banks -> rows at the same place in the period get distinct XOR values
 template <int PITCH>
 __device__ __forceinline__ int swz_k(int row) { return PITCH == 128 ? (row >> 1) & 7 : (row >> 2) & 3; }
-// 512-byte rows read with ds_read_b64_tr_b16 (4 consecutive k x 64 contiguous bytes)
-__device__ __forceinline__ int swz512(int row) { return (row & 3) << 2; }
 
-// T = element type of A, B, C, D (_Float16 or float); BKB = bytes of a K-contiguous tile row (64 halves or 32 floats at
-// 128).  blockIdx.y = problem of a batch.  4 waves of 128 x 128, one per SIMD.
-template <class T, bool NN, int BKB>
+// The fp32 kernel (TN only), on v_mfma_f32_32x32x2_f32: 4 x 4 blocks of 32 x 32 per wave.  BKB = bytes of a K-contiguous
+// tile row (32 floats at 128).  blockIdx.y = problem of a batch.  4 waves of 128 x 128, one per SIMD.
+template <int BKB>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restrict__ Cin, T *__restrict__ D, int M, int N,
-            int K, float alpha, float beta) {
-  constexpr bool F32 = sizeof(T) == 4;
+gemm_kernel_f32(const float *__restrict__ A, const float *__restrict__ B, const float *__restrict__ Cin, float *__restrict__ D,
+                int M, int N, int K, float alpha, float beta) {
+  using T = float;
   constexpr int ES = sizeof(T);
   constexpr int BK = BKB / ES;
-  static_assert(!(F32 && NN), "the N-contiguous B layout is built for fp16 only");
-  using Frag = std::conditional_t<F32, f32x4, half8>;  // 16 bytes of a row: the operand of one K-step
+  using Frag = f32x4;  // 16 bytes of a row: the operand of one K-step
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -68,7 +65,7 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   constexpr int WN = 2, NWAVES = 4;
   constexpr int NB = 4;                // 32-column blocks per wave
   constexpr int PITCH = BKB;           // bytes per K-contiguous LDS row
-  constexpr int A_TILE = BM * PITCH;   // TN: B tile likewise (n rows); NN: BK rows (k) of 512 B
+  constexpr int A_TILE = BM * PITCH;   // B tile likewise (n rows)
   constexpr int STAGE = 2 * A_TILE;
   constexpr int CPW = A_TILE / 1024 / NWAVES;  // 16-byte pieces per lane and operand tile
   constexpr int RPC = 1024 / PITCH;    // rows per wave-wide 1 KB piece
@@ -95,7 +92,7 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   D += batch * M * N;
   if (Cin) Cin += batch * M * N;
   const char *Ap = (const char *)(A + (int64_t)m0 * K);
-  const char *Bp = NN ? (const char *)(B + n0) : (const char *)(B + (int64_t)n0 * K);
+  const char *Bp = (const char *)(B + (int64_t)n0 * K);
 
   // ---- global -> register -> LDS staging, 16 B per lane and piece.  Piece i of wave w covers tile rows
   // (i*NWAVES + w)*RPC .. +RPC; lane l owns LDS slot (row l / CPR, chunk position l % CPR) of the piece and fetches
@@ -109,13 +106,7 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
     const int row = (i * NWAVES + wave) * RPC + lane / (PITCH / 16);
     const int cp = lane % (PITCH / 16);
     goff_a[i] = (uint32_t)row * (uint32_t)(K * ES) + (uint32_t)((cp ^ swz_k<PITCH>(row)) * 16);
-    if (!NN) {
-      goff_b[i] = goff_a[i];
-    } else {  // B tile is BK rows (k) of 512 B (256 n): 2 rows per piece
-      const int krow = (i * NWAVES + wave) * 2 + (lane >> 5);
-      const int cpb = lane & 31;
-      goff_b[i] = (uint32_t)krow * (uint32_t)(N * 2) + (uint32_t)((cpb ^ swz512(krow)) * 16);
-    }
+    goff_b[i] = goff_a[i];
   }
   const uint32_t st_off = wave * 1024 + lane * 16;  // + (piece * NWAVES) * 1024 (+ A_TILE for B) + stage * STAGE
   int4v stg[2 * CPW];                               // the tile in flight: A pieces, then B pieces
@@ -124,7 +115,7 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   using Rsrc = __amdgpu_buffer_rsrc_t;
   auto tile_ptrs = [&](int kt, Rsrc &ga, Rsrc &gb) {
     const char *pa = Ap + (size_t)kt * PITCH;
-    const char *pb = NN ? Bp + (size_t)kt * BK * (size_t)(N * 2) : Bp + (size_t)kt * PITCH;
+    const char *pb = Bp + (size_t)kt * PITCH;
     ga = __builtin_amdgcn_make_buffer_rsrc((void *)pa, 0, -1, 0x00020000);
     gb = __builtin_amdgcn_make_buffer_rsrc((void *)pb, 0, -1, 0x00020000);
   };
@@ -147,17 +138,6 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
     a_rd[s] = (wm * 128 + r) * PITCH + (((2 * s + g) ^ swz_k<PITCH>(r)) * 16);               // + 32 rows per m block
     b_rd[s] = A_TILE + (wn * NB * 32 + r) * PITCH + (((2 * s + g) ^ swz_k<PITCH>(r)) * 16);  // + 32 rows per n block (TN)
   }
-  // NN: B^T operand via ds_read_b64_tr_b16 from [k][n] rows (see the V operand of the attention kernel)
-  const int li = lane & 15;
-  const int bk_row = 8 * g + (li >> 2);                                // + 16 s + 4 h2: slot t of lane g is k = 16s + 8g + t, as in A
-  const int bn_col = wn * NB * 32 + 16 * ((lane >> 4) & 1) + 4 * (li & 3);  // + 32 nb
-  int bt_rd[NB];
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int c = (bn_col + 32 * nb) >> 3;
-    bt_rd[nb] = A_TILE + bk_row * 512 + ((c ^ swz512(bk_row)) * 16) + (bn_col & 7) * 2;
-  }
-
   f32x16 acc[4][NB];
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb)
@@ -174,30 +154,15 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
     const int blk = i == 0 ? 0 : i == 1 ? 0 : i <= 4 ? i - 1 : i - 4;
     if (is_a) {
       aop[blk] = *(const Frag *)(st + a_rd[s] + blk * 32 * PITCH);
-    } else if (!NN) {
-      bop[blk] = *(const Frag *)(st + b_rd[s] + blk * 32 * PITCH);
     } else {
-      if constexpr (!F32) {
-        union {
-          struct { short4v lo, hi; } p;
-          half8 h;
-        } u;
-        const char *bp = st + bt_rd[blk] + s * 16 * 512;
-        u.p.lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp));
-        u.p.hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(short4v, bp + 4 * 512));
-        bop[blk] = u.h;
-      }
+      bop[blk] = *(const Frag *)(st + b_rd[s] + blk * 32 * PITCH);
     }
   };
   // One block multiply (one MFMA, or 4 for fp32 operands).  Transposed block: MFMA rows = n (B operand first)
   auto mma_block = [&](const Frag (&aop)[4], const Frag (&bop)[NB], int mb, int nb) {
-    if constexpr (F32) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(bop[nb][e], aop[mb][e], acc[mb][nb], 0, 0, 0);
-    } else {
-      acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bop[nb], aop[mb], acc[mb][nb], 0, 0, 0);
-    }
+    for (int e = 0; e < 4; ++e)
+      acc[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x2f32(bop[nb][e], aop[mb][e], acc[mb][nb], 0, 0, 0);
   };
 
   // Pipeline: two LDS stages and one tile in registers.  While tile kt multiplies out of stage kt % 2, the registers
@@ -270,7 +235,7 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
   constexpr int E_PITCH = 128 * 4 + 16;          // bytes per staged row of 128 floats, padded
   constexpr int EPL = 16 / ES;                   // elements per lane and store (8 halves / 4 floats)
   constexpr int LPR = 128 / EPL, RPP = 64 / LPR; // lanes per row, rows per wave-wide store
-  using OutV = std::conditional_t<F32, f32x4, half8>;
+  using OutV = f32x4;
   const bool with_c = Cin != nullptr && beta != 0.f;
   char *et = smem + wave * (32 * E_PITCH);
   const int e_row = lane / LPR, e_col = (lane % LPR) * EPL;
@@ -320,9 +285,9 @@ gemm_kernel(const T *__restrict__ A, const T *__restrict__ B, const T *__restric
 __device__ __forceinline__ int swz512n(int row) { return ((row & 3) | (((row >> 3) & 1) << 2)) << 1; }
 
 // The fp16 kernel on 16x16x32 MFMAs (v_mfma_f32_16x16x32_f16): the same workgroup tile, staging path and epilogue as
-// gemm_kernel, with the wave's 128 x 128 of C as 8 x 8 blocks (NWAVES = 4; NWAVES = 8 runs two waves per SIMD on
+// gemm_kernel_f32, with the wave's 128 x 128 of C as 8 x 8 blocks (NWAVES = 4; NWAVES = 8 runs two waves per SIMD on
 // 128 x 64 each and measured the same).  Measured, 8192^3 TN, same session: 1401 TFLOP/s on U(-1,1) operands against
-// 1309 for gemm_kernel<_Float16> (8 waves: 1390); on constant operands 1837 against 2048 (LDS writes between the
+// 1309 for the same kernel on 32x32x16 MFMAs (8 waves: 1390); on constant operands 1837 against 2048 (LDS writes between the
 // short multiplies hold the MFMA pipe up for about 20 cycles each).  On U(-1,1) operands this board is
 // power-limited and the deeper, narrower MFMA moves half the accumulator bits per FLOP: a register-only loop sustains
 // 1.90 PFLOP/s with it against 1.69 with 32x32x16.  Lane (c = lane % 16, g = lane / 16) holds, of an operand fragment,
@@ -349,7 +314,7 @@ gemm_kernel16(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, co
   constexpr int KS = PITCH / 64;       // K-steps per tile: 64 bytes of a row (four 16-byte fragments, one per g) each
   const int wm = wave / WN, wn = wave % WN;
 
-  // tile order and XCD remap as in gemm_kernel
+  // tile order and XCD remap as in gemm_kernel_f32
   const int tiles_n = N / BN, tiles_m = M / BM;
   int t = xcd_remap(blockIdx.x, gridDim.x);
   constexpr int GROUP = 8;
@@ -370,7 +335,7 @@ gemm_kernel16(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, co
   const char *Ap = (const char *)(A + (int64_t)m0 * K);
   const char *Bp = NN ? (const char *)(B + n0) : (const char *)(B + (int64_t)n0 * K);
 
-  // ---- global -> register -> LDS staging (see gemm_kernel)
+  // ---- global -> register -> LDS staging (see gemm_kernel_f32)
   uint32_t goff_a[CPW], goff_b[CPW];
 #pragma unroll
   for (int i = 0; i < CPW; ++i) {
@@ -448,7 +413,7 @@ gemm_kernel16(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, co
     }
   };
 
-  // Pipeline as in gemm_kernel (two LDS stages, one tile in registers, one barrier per tile), laid out as slots of
+  // Pipeline as in gemm_kernel_f32 (two LDS stages, one tile in registers, one barrier per tile), laid out as slots of
   // one multiply each (K-step major, then m block, then n block; SPM = NBN slots per m block) with at most one piece
   // of other work behind each multiply, pinned in that order.  Fragment registers: the n-side fragments of a K-step
   // are live throughout it and double-buffered (bop[K-step parity]); the m-side fragment of block mb is only needed
@@ -522,7 +487,7 @@ gemm_kernel16(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, co
   // the dependency through the asm statements)
   asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
   // ---- epilogue: D = alpha * acc + beta * C in fp32, each 16 x 128 row of blocks staged through the wave's own LDS
-  // region (see gemm_kernel) and stored as whole rows, 16 bytes per lane
+  // region (see gemm_kernel_f32) and stored as whole rows, 16 bytes per lane
   constexpr int E_PITCH = 128 * 4 + 16;
   constexpr int EPL = 8;                          // halves per lane and store
   constexpr int WCOLS = NBN * 16;                   // columns of the wave tile
@@ -571,7 +536,7 @@ struct GemmLaunch {
   static constexpr int WAVES16 = 4;  // waves of the fp16 kernel
   static constexpr auto kern = [] {
     if constexpr (sizeof(T) == 2) return gemm_kernel16<NN, WAVES16>;
-    else return gemm_kernel<T, NN, BKB>;
+    else return gemm_kernel_f32<BKB>;
   }();
   // one-time set-up, thread-safe and callable ahead of any launch
   static hipError_t prepare() {
