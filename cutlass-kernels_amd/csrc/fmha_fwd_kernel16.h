@@ -138,13 +138,16 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   float m_ref[QB], m_lane[QB], thr_raw[QB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) m_ref[qb] = -INFINITY, m_lane[qb] = -INFINITY, thr_raw[qb] = -INFINITY;
-  // The row sum is taken on the MFMA pipe (the VALU issue slots are the scarce resource with four-pass MFMAs): an
-  // all-ones A operand times P^T gives every output row the sum over the K-step's 32 keys of the lane's query, summed
-  // over P as rounded to fp16 (the weights the second GEMM applies), in fp32, complete across lanes.
+  // Row sum: with v_dot2_f32_f16 over this lane's quarter of each query's keys (l_run), or -- head dim 64, which has
+  // the twelve registers to spare and gains 2 % from it -- on the MFMA pipe: an all-ones A operand times P^T gives
+  // every output row the sum over the K-step's 32 keys of the lane's query, complete across lanes (l_acc).  Both sum
+  // P as rounded to fp16, the weights the second GEMM applies, in fp32.
+  constexpr bool MFMA_SUM = D == 64;
+  float l_run[QB];
   f32x4 l_acc[QB];
-#pragma unroll
-  for (int qb = 0; qb < QB; ++qb) l_acc[qb] = f32x4{0.f, 0.f, 0.f, 0.f};
   half8 ones;
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) l_run[qb] = 0.f, l_acc[qb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int t = 0; t < 8; ++t) ones[t] = (_Float16)1.0f;
   const float inv_c = 1.0f / c_log2;
@@ -200,7 +203,8 @@ fmha_fwd_kernel16(const FmhaArgs a) {
         const float alpha = __builtin_amdgcn_exp2f(m_ref[qb] - m_new);
         m_ref[qb] = m_new;
         thr_raw[qb] = (m_new + kTau) * inv_c;
-        l_acc[qb] *= alpha;
+        l_run[qb] *= alpha;
+        if constexpr (MFMA_SUM) l_acc[qb] *= alpha;
 #pragma unroll
         for (int db = 0; db < DB; ++db) oacc[db][qb] *= alpha;
       }
@@ -208,20 +212,36 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   };
   // P = exp2(c*S - m_ref), cast to fp16 in the B-operand register order of the second GEMM
   auto softmax_exp = [&](const f32x4 (&sacc)[KB][QB], half8 (&pb)[QB][PS]) {
+    const half2v one2 = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb)
+    for (int qb = 0; qb < QB; ++qb) {
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
         for (int t = 0; t < 4; ++t)
           pb[qb][kb / 2][4 * (kb % 2) + t] = (_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][qb][t], c_log2, -m_ref[qb]));
+      if constexpr (!MFMA_SUM) {
+        float rs = 0.f, rs2 = 0.f;
+#pragma unroll
+        for (int ps = 0; ps < PS; ++ps)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const half2v pp = {pb[qb][ps][2 * t], pb[qb][ps][2 * t + 1]};
+            if (t & 1) rs2 = __builtin_amdgcn_fdot2(pp, one2, rs2, false);
+            else rs = __builtin_amdgcn_fdot2(pp, one2, rs, false);
+          }
+        l_run[qb] += rs + rs2;
+      }
+    }
   };
   // O^T += V^T . P^T for the V tile at LDS byte offset vt
   auto pv = [&](uint32_t vt, const half8 (&pb)[QB][PS]) {
+    if constexpr (MFMA_SUM) {
 #pragma unroll
-    for (int ps = 0; ps < PS; ++ps)
+      for (int ps = 0; ps < PS; ++ps)
 #pragma unroll
-      for (int qb = 0; qb < QB; ++qb) l_acc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb[qb][ps], l_acc[qb], 0, 0, 0);
+        for (int qb = 0; qb < QB; ++qb) l_acc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb[qb][ps], l_acc[qb], 0, 0, 0);
+    }
 #pragma unroll
     for (int ps = 0; ps < PS; ++ps)
 #pragma unroll
@@ -373,7 +393,14 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   // loop's last barrier) and leaves as whole rows, 16 bytes per lane.
   float l_tot[QB];
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) l_tot[qb] = l_acc[qb][0];
+  for (int qb = 0; qb < QB; ++qb) {
+    if constexpr (MFMA_SUM) {
+      l_tot[qb] = l_acc[qb][0];
+    } else {
+      l_tot[qb] = l_run[qb] + __shfl_xor(l_run[qb], 16, 64);
+      l_tot[qb] += __shfl_xor(l_tot[qb], 32, 64);
+    }
+  }
   {
     char *ot = smem + wave * (32 * C::O_PITCH);
 #pragma unroll
