@@ -26,7 +26,9 @@ def run_case(spec):
         q16, k16, v16 = (x.astype(np.float16) for x in (q, k, v))
         plan = f.fmha_forward_plan(f.CFK_FP16, B, H, S, Skv, D)
         mfma = f.fmha_forward_mfma(f.CFK_FP16, B, H, S, Skv, D)
-        o = pkg.fmha_forward(to_dev(q16), to_dev(k16), to_dev(v16))
+        rm = torch.full((B, H, S), -1.0, dtype=torch.float32, device="cuda:0")
+        rs = torch.full((B, H, S), -1.0, dtype=torch.float32, device="cuda:0")
+        o = pkg.fmha_forward(to_dev(q16), to_dev(k16), to_dev(v16), row_max=rm, row_sum=rs)
         qf, kf, vf = (x.astype(np.float32) for x in (q16, k16, v16))
     else:
         (qc, qs), (kc, ks) = oracle.quantize_e4m3_per_tensor(q), oracle.quantize_e4m3_per_tensor(k)
@@ -51,7 +53,15 @@ def run_case(spec):
                          out=ref)
     sel = ~np.isnan(ref)
     _, pct = oracle.verify_tensor(got[sel], ref[sel])
-    return dict(case=spec, block_m=plan[0], block_n=plan[1], mfma=mfma, lds_bytes=plan[2], checked=int(sel.sum()),
+    taps = None
+    if mode == "f16":
+        # the row-max / row-sum taps of the first and last (batch, head): log2-domain max, sum not reciprocal
+        st = oracle.attention_f32(qf, kf, vf, bh_pairs=pairs, want_stats=True)
+        m_ref, inv_ref = st["row_max"], st["inv_sum"]
+        ok = ~np.isnan(m_ref)
+        mi = rm.cpu().numpy() / oracle.LOG2E
+        taps = [float(np.abs(mi[ok] - m_ref[ok]).max()), float(np.abs(1.0 / rs.cpu().numpy()[ok] / inv_ref[ok] - 1.0).max())]
+    return dict(taps=taps, case=spec, block_m=plan[0], block_n=plan[1], mfma=mfma, lds_bytes=plan[2], checked=int(sel.sum()),
                 max_abs=max_abs(got[sel], ref[sel]), err_pct=pct, nan=bool(np.isnan(got).any()))
 
 
