@@ -21,7 +21,7 @@
  * exp-branch == exp2-branch, rows of P sum to one, Q = 0 gives the mean of V, a dominant key selects
  * its V row, key-permutation invariance, integer-valued inputs give bit-exact scores.
  * The reference holds no golden vectors for this path; the literal curand input stream of its driver
- * is not reproducible here ("parity unpinned" for that stream only -- see the design notes).
+ * is not reproducible here ("parity unpinned" for that stream only: the tests draw their own seeded inputs).
  */
 #include <math.h>
 #include <stdint.h>
