@@ -41,6 +41,18 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     assert plans("256x128") == "(256, 128) (128, 32) (256, 128) (128, 64)"     # no such tile at head dim 256; 384 % 256 != 0
     assert plans("large") == "(256, 64) (128, 32) (256, 64) (128, 64)"
     assert plans("128x128") == "(128, 128) (128, 32) (128, 128) (128, 128)"
+    # the MFMA shape suffix: served for fp16 at head dims 64/128 only (e4m3 and head dim 256 ignore the wish)
+    mfma_code = ("import sys; sys.path.insert(0, %r); import __graft_entry__ as e; p = e.load_package(); f = p.fmha; "
+                 "print(f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 512, 512, 128), f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 512, 512, 64), "
+                 "f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 512, 512, 256), f.fmha_forward_mfma(f.CFK_FP8_E4M3, 2, 4, 512, 512, 128), "
+                 "f.fmha_forward_plan(f.CFK_FP16, 2, 4, 512, 512, 128)[:2])" % ROOT)
+    def shapes(wish):
+        env = dict(os.environ, CFK_FMHA_TILE=wish)
+        return subprocess.run([sys.executable, "-c", mfma_code], env=env, capture_output=True, text=True, check=True).stdout.strip()
+    assert shapes("128x64/16") == "16 16 32 32 (128, 64)"
+    assert shapes("256x64/16") == "16 32 32 32 (256, 64)"      # no 256-row 16x16x32 build at head dim 64
+    assert shapes("256x64/32") == "32 32 32 32 (256, 64)"
+    assert shapes("128x64") == "32 32 32 32 (128, 64)"
     assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:2] == (256, 64)   # big problem: automatic choice
     # ... on 16x16x32 MFMAs for fp16 at head dims 64 and 128; small problems, head dim 256 and e4m3 stay on 32x32
     assert f.fmha_forward_mfma(f.CFK_FP16, 8, 16, 2048, 2048, 128) == 16
