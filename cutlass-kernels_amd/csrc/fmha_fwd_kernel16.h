@@ -1,14 +1,16 @@
-// The fp16 FMHA forward kernel on 16x16x32 MFMAs (v_mfma_f32_16x16x32_f16).  Same algorithm, pipeline forms, LDS
-// staging and epilogue as fmha_fwd_kernel.h (which it takes its configuration struct and host-side plumbing from);
-// what differs is the MFMA shape and with it every register layout.
+// The fp16 FMHA forward kernel on 16x16x32 MFMAs (v_mfma_f32_16x16x32_f16).  Same algorithm, LDS staging, pipeline
+// (the plain one-tile-per-barrier form) and epilogue as fmha_fwd_kernel.h, which it takes its configuration struct and
+// host-side plumbing from; what differs is the MFMA shape, with it every register layout, and how the softmax notices
+// that its reference point has to move: not by a row max per tile but by the row sum it needs anyway (softmax_tile
+// below; 22 VALU instructions per wave and tile less, +3..6 % on N(0,1) data, results bit-identical).
 //
 // Why a second shape: on N(0,1) data this board is power-limited, and a register-only loop of 16x16x32 MFMAs sustains
 // 1.89-1.90 PFLOP/s there against 1.69 for 32x32x16 (2.39 against 2.47 on constant operands): a multiply that is
 // twice as deep per accumulator element moves half the accumulator bits per FLOP.  Measured on N(0,1) tensors against
-// the 32x32 kernel: B=8 H=16 S=2048 D=128 1107 against 1078 TFLOP/s, B=4 H=32 S=4096 D=64 919 against 875; on constant
-// tensors, where nothing limits the clock, the 32x32 kernel is the faster one (1480 against 1244): twice the MFMA
-// instructions for the same VALU work leave fewer issue slots.  Head dim 256 gains nothing (929 against 932) and
-// keeps the 32x32 kernel.
+// the 32x32 kernel, both with a row max per tile: B=8 H=16 S=2048 D=128 1107 against 1078 TFLOP/s, B=4 H=32 S=4096 D=64
+// 919 against 875; on constant tensors, where nothing limits the clock, the 32x32 kernel is the faster one (1480
+// against 1244): twice the MFMA instructions for the same VALU work leave fewer issue slots.  Head dim 256 gains
+// nothing (929 against 932) and keeps the 32x32 kernel.
 //
 // Layouts (lane = 16 g + c, c = 0..15, g = 0..3):
 //   A operand: row c of the 16-row block, contraction slots 8g .. 8g+7;   B operand: column c, slots 8g .. 8g+7;
@@ -133,85 +135,62 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) oacc[db][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  // per query block: softmax reference point; this lane's running max of the raw scores (a quarter of the query's
-  // keys); running sum; raw-score threshold (m_ref + tau) / c above which the reference point moves
-  float m_ref[QB], m_lane[QB], thr_raw[QB];
+  // per query block: softmax reference point (log2 domain); this lane's running max of the raw scores (a quarter of
+  // the query's keys), kept for the taps only
+  float m_ref[QB], m_lane[QB];
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) m_ref[qb] = -INFINITY, m_lane[qb] = -INFINITY, thr_raw[qb] = -INFINITY;
-  // Row sum: with v_dot2_f32_f16 over this lane's quarter of each query's keys (l_run), or -- head dim 64, which has
-  // the twelve registers to spare and gains 2 % from it -- on the MFMA pipe: an all-ones A operand times P^T gives
-  // every output row the sum over the K-step's 32 keys of the lane's query, complete across lanes (l_acc).  Both sum
-  // P as rounded to fp16, the weights the second GEMM applies, in fp32.
-  constexpr bool MFMA_SUM = D == 64;
+  for (int qb = 0; qb < QB; ++qb) m_ref[qb] = -INFINITY, m_lane[qb] = -INFINITY;
+  // Row sum: v_dot2_f32_f16 over this lane's quarter of each query's keys, of P as rounded to fp16 (the weights the
+  // second GEMM applies), in fp32; the four quarters meet in the epilogue.
   float l_run[QB];
-  f32x4 l_acc[QB];
-  half8 ones;
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) l_run[qb] = 0.f, l_acc[qb] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int t = 0; t < 8; ++t) ones[t] = (_Float16)1.0f;
-  const float inv_c = 1.0f / c_log2;
+  for (int qb = 0; qb < QB; ++qb) l_run[qb] = 0.f;
 
-  constexpr int NPRE = C::KPRE;
-  half8 kpre[NPRE ? NPRE : 1];
-  auto read_kfrag = [&](uint32_t kt, int s, int kb) -> half8 { return *LDS_AT(half8, kt + k_rd[s] + kb * 16 * C::K_PITCH); };
-  // the first NPRE fragments (order: K-step major, key block minor) of the K tile in slot `stage`
-  auto prefetch_k = [&](int stage) {
-#pragma unroll
-    for (int f = 0; f < NPRE; ++f) kpre[f] = read_kfrag(stage * C::K_TILE, f / KB, f % KB);
-  };
+  static_assert(C::KPRE == 0 && C::SUB == 1, "one key tile per barrier, no K fragment prefetch in this kernel");
+  const float sum_cap = __builtin_amdgcn_exp2f(kTau);
+  const bool want_taps = a.row_max != nullptr || a.row_sum != nullptr;
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
   // S^T = K . Q^T for the K tile in LDS slot `stage`
-  auto qk = [&](int stage, f32x4 (&sacc)[KB][QB], bool use_pre = false) {
+  auto qk = [&](int stage, f32x4 (&sacc)[KB][QB]) {
     const uint32_t kt = stage * C::K_TILE;
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) sacc[kb][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < KS; ++s)
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
-        half8 ka;
-        if (use_pre && s * KB + kb < NPRE) ka = kpre[s * KB + kb];
-        else ka = read_kfrag(kt, s, kb);
+        const half8 ka = *LDS_AT(half8, kt + k_rd[s] + kb * 16 * C::K_PITCH);
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) sacc[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qreg[qb][s], sacc[kb][qb], 0, 0, 0);
+        for (int qb = 0; qb < QB; ++qb)
+          sacc[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qreg[qb][s], s == 0 ? zero4 : sacc[kb][qb], 0, 0, 0);
       }
   };
-  // Row max of a finished S tile and the deferred rescale (online_softmax.h:123-165).  A lane only tests its own
-  // quarter of each query's keys against the threshold; the (rare, wave-uniform) slow path completes the max.
-  auto row_max_and_rescale = [&](const f32x4 (&sacc)[KB][QB]) {
-    float mx[QB];
-    bool over = false;
+  // this lane's max over its quarter of the keys of query block qb: a chain of three-operand maxima
+  auto lane_max = [&](const f32x4 (&sacc)[KB][QB], int qb) -> float {
+    float mx = __builtin_fmaxf(sacc[0][qb][0], sacc[0][qb][1]);
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int t = kb ? 0 : 2; t < 4; t += 2) mx = __builtin_fmaxf(__builtin_fmaxf(mx, sacc[kb][qb][t]), sacc[kb][qb][t + 1]);
+    return mx;
+  };
+  // Move the reference point of every query up to the row max of `sacc` (if that is above it) and re-base O and l
+  // (online_softmax.h:123-165); for the first tile the old reference point is -inf and O and l are zero.
+  auto rebase = [&](const f32x4 (&sacc)[KB][QB]) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-      // a chain of three-operand maxima, two new scores each
-      mx[qb] = __builtin_fmaxf(sacc[0][qb][0], sacc[0][qb][1]);
+      const float mx = lane_max(sacc, qb);
+      float mfull = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mfull = fmaxf(mfull, __shfl_xor(mfull, 32, 64));
+      const float m_new = fmaxf(m_ref[qb], mfull * c_log2);
+      const float alpha = __builtin_amdgcn_exp2f(m_ref[qb] - m_new);
+      m_ref[qb] = m_new;
+      l_run[qb] *= alpha;
 #pragma unroll
-      for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-        for (int t = kb ? 0 : 2; t < 4; t += 2) mx[qb] = __builtin_fmaxf(__builtin_fmaxf(mx[qb], sacc[kb][qb][t]), sacc[kb][qb][t + 1]);
-      m_lane[qb] = __builtin_fmaxf(m_lane[qb], mx[qb]);
-      over = over || mx[qb] > thr_raw[qb];
-    }
-    if (__builtin_amdgcn_ballot_w64(over) != 0) {
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        float mfull = fmaxf(mx[qb], __shfl_xor(mx[qb], 16, 64));
-        mfull = fmaxf(mfull, __shfl_xor(mfull, 32, 64)) * c_log2;
-        const float m_new = fmaxf(m_ref[qb], mfull);
-        const float alpha = __builtin_amdgcn_exp2f(m_ref[qb] - m_new);
-        m_ref[qb] = m_new;
-        thr_raw[qb] = (m_new + kTau) * inv_c;
-        l_run[qb] *= alpha;
-        if constexpr (MFMA_SUM) l_acc[qb] *= alpha;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) oacc[db][qb] *= alpha;
-      }
+      for (int db = 0; db < DB; ++db) oacc[db][qb] *= alpha;
     }
   };
-  // P = exp2(c*S - m_ref), cast to fp16 in the B-operand register order of the second GEMM
-  auto softmax_exp = [&](const f32x4 (&sacc)[KB][QB], half8 (&pb)[QB][PS]) {
+  // P = exp2(c*S - m_ref), cast to fp16 in the B-operand register order of the second GEMM, and the tile's row sums of
+  // P as rounded (the weights the second GEMM applies), in fp32
+  auto exp_and_sum = [&](const f32x4 (&sacc)[KB][QB], half8 (&pb)[QB][PS], float (&rsum)[QB]) {
     const half2v one2 = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -220,28 +199,53 @@ fmha_fwd_kernel16(const FmhaArgs a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
           pb[qb][kb / 2][4 * (kb % 2) + t] = (_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][qb][t], c_log2, -m_ref[qb]));
-      if constexpr (!MFMA_SUM) {
-        float rs = 0.f, rs2 = 0.f;
-#pragma unroll
-        for (int ps = 0; ps < PS; ++ps)
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const half2v pp = {pb[qb][ps][2 * t], pb[qb][ps][2 * t + 1]};
-            if (t & 1) rs2 = __builtin_amdgcn_fdot2(pp, one2, rs2, false);
-            else rs = __builtin_amdgcn_fdot2(pp, one2, rs, false);
-          }
-        l_run[qb] += rs + rs2;
-      }
-    }
-  };
-  // O^T += V^T . P^T for the V tile at LDS byte offset vt
-  auto pv = [&](uint32_t vt, const half8 (&pb)[QB][PS]) {
-    if constexpr (MFMA_SUM) {
+      float rs = 0.f, rs2 = 0.f;
 #pragma unroll
       for (int ps = 0; ps < PS; ++ps)
 #pragma unroll
-        for (int qb = 0; qb < QB; ++qb) l_acc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb[qb][ps], l_acc[qb], 0, 0, 0);
+        for (int t = 0; t < 4; ++t) {
+          const half2v pp = {pb[qb][ps][2 * t], pb[qb][ps][2 * t + 1]};
+          if (t & 1) rs2 = __builtin_amdgcn_fdot2(pp, one2, rs2, false);
+          else rs = __builtin_amdgcn_fdot2(pp, one2, rs, false);
+        }
+      rsum[qb] = rs + rs2;
     }
+  };
+  // The softmax of key tile jt.  No row max is taken in the common case: a weight that leaves the fp16 range (or
+  // merely exceeds 2^tau) shows in the row sum, which is needed anyway.  An infinite or large sum sends the wave to
+  // the (wave-uniform, rare) slow path: the scores are gone by then (the exponentials overwrote them; keeping them
+  // would cost 32 registers), so it recomputes them with K fragments fetched straight from global memory, moves the
+  // reference point up to their row max and takes the exponentials again.
+  auto softmax_tile = [&](int jt, const f32x4 (&sacc)[KB][QB], half8 (&pb)[QB][PS]) {
+    if (want_taps) {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) m_lane[qb] = __builtin_fmaxf(m_lane[qb], lane_max(sacc, qb));
+    }
+    float rsum[QB];
+    exp_and_sum(sacc, pb, rsum);
+    bool over = false;
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) over = over || !(rsum[qb] < sum_cap);
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(over) != 0, 0)) {
+      f32x4 sr[KB][QB];
+      const char *kt = Kp + (size_t)jt * ((size_t)BN * k_ld) + (size_t)c * k_ld + 16 * g;
+#pragma unroll
+      for (int s = 0; s < KS; ++s)
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          const half8 ka = *(const half8 *)(kt + (size_t)(16 * kb) * k_ld + 64 * s);
+#pragma unroll
+          for (int qb = 0; qb < QB; ++qb)
+            sr[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qreg[qb][s], s == 0 ? zero4 : sr[kb][qb], 0, 0, 0);
+        }
+      rebase(sr);
+      exp_and_sum(sr, pb, rsum);
+    }
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) l_run[qb] += rsum[qb];
+  };
+  // O^T += V^T . P^T for the V tile at LDS byte offset vt
+  auto pv = [&](uint32_t vt, const half8 (&pb)[QB][PS]) {
 #pragma unroll
     for (int ps = 0; ps < PS; ++ps)
 #pragma unroll
@@ -258,8 +262,8 @@ fmha_fwd_kernel16(const FmhaArgs a) {
       }
   };
 
-  // The three step forms of fmha_fwd_kernel.h (see there for the slot bookkeeping): plain, two tiles per barrier,
-  // K fragment prefetch.
+  // One pipeline step for tile j (parity P = j & 1), as in fmha_fwd_kernel.h: on entry s_cur = S_j is finished, K_{j+1}
+  // sits in K stage P^1 and V_j in V stage P.
   auto step = [&](auto parity, auto has_next, int j, f32x4 (&s_cur)[KB][QB], f32x4 (&s_nxt)[KB][QB]) {
     constexpr int P = decltype(parity)::value;
     constexpr bool HAS_NEXT = decltype(has_next)::value;
@@ -267,125 +271,32 @@ fmha_fwd_kernel16(const FmhaArgs a) {
     load_v(j + 1 < n_tiles ? j + 1 : n_tiles - 1, P ^ 1);
     half8 pb[QB][PS];
     if (HAS_NEXT) qk(P ^ 1, s_nxt);
-    softmax_exp(s_cur, pb);
+    softmax_tile(j, s_cur, pb);
     pv(P * C::V_TILE, pb);
-    if (HAS_NEXT) row_max_and_rescale(s_nxt);
-    wait_lds_dma();
-    __syncthreads();
-  };
-  auto step2 = [&](auto parity, auto last, int J, f32x4 (&s_a)[KB][QB], f32x4 (&s_b)[KB][QB]) {
-    constexpr int P = decltype(parity)::value;
-    constexpr bool LAST = decltype(last)::value;
-    const int t0 = 2 * J, t_max = n_tiles - 1;
-    load_k(t0 + 3 < t_max ? t0 + 3 : t_max, (2 * P + 3) % 4);
-    load_k(t0 + 4 < t_max ? t0 + 4 : t_max, (2 * P) % 4);
-    {
-      half8 pb[QB][PS];
-      qk((2 * P + 1) % 4, s_b);
-      softmax_exp(s_a, pb);
-      pv(((2 * P) % 4) * C::V_TILE, pb);
-      row_max_and_rescale(s_b);
-    }
-    load_v(t0 + 2 < t_max ? t0 + 2 : t_max, (2 * P + 2) % 4);
-    load_v(t0 + 3 < t_max ? t0 + 3 : t_max, (2 * P + 3) % 4);
-    {
-      half8 pb[QB][PS];
-      if (!LAST) qk((2 * P + 2) % 4, s_a);
-      softmax_exp(s_b, pb);
-      pv(((2 * P + 1) % 4) * C::V_TILE, pb);
-      if (!LAST) row_max_and_rescale(s_a);
-    }
-    wait_lds_dma();
-    __syncthreads();
-  };
-  auto step_p = [&](auto jmod4, auto has_next, int j, f32x4 (&s_cur)[KB][QB], f32x4 (&s_nxt)[KB][QB]) {
-    constexpr int J4 = decltype(jmod4)::value;
-    constexpr int P = J4 & 1;
-    constexpr bool HAS_NEXT = decltype(has_next)::value;
-    half8 pb[QB][PS];
-    if (HAS_NEXT) qk((J4 + 1) % 4, s_nxt, true);
-    load_k(j + 3 < n_tiles ? j + 3 : n_tiles - 1, (J4 + 3) % 4);
-    load_v(j + 1 < n_tiles ? j + 1 : n_tiles - 1, P ^ 1);
-    softmax_exp(s_cur, pb);
-    pv(P * C::V_TILE, pb);
-    if (HAS_NEXT) {
-      prefetch_k((J4 + 2) % 4);
-      row_max_and_rescale(s_nxt);
-    }
     wait_lds_dma();
     __syncthreads();
   };
 
   using std::integral_constant;
   f32x4 s_a[KB][QB], s_b[KB][QB];
-  if constexpr (C::KPRE > 0) {
-    using T = integral_constant<bool, true>;
-    using F = integral_constant<bool, false>;
-    const int t_max = n_tiles - 1;
-    load_k(0, 0);
-    load_v(0, 0);
-    load_k(1, 1);
-    load_k(2 < t_max ? 2 : t_max, 2);
-    wait_lds_dma();
-    __syncthreads();
-    qk(0, s_a);
-    prefetch_k(1);
-    row_max_and_rescale(s_a);
-    int j = 0;
-    for (; j + 4 < n_tiles; j += 4) {
-      step_p(integral_constant<int, 0>{}, T{}, j, s_a, s_b);
-      step_p(integral_constant<int, 1>{}, T{}, j + 1, s_b, s_a);
-      step_p(integral_constant<int, 2>{}, T{}, j + 2, s_a, s_b);
-      step_p(integral_constant<int, 3>{}, T{}, j + 3, s_b, s_a);
-    }
-    step_p(integral_constant<int, 0>{}, T{}, j, s_a, s_b);
-    step_p(integral_constant<int, 1>{}, T{}, j + 1, s_b, s_a);
-    step_p(integral_constant<int, 2>{}, T{}, j + 2, s_a, s_b);
-    step_p(integral_constant<int, 3>{}, F{}, j + 3, s_b, s_a);
-  } else if constexpr (C::SUB == 2) {
-    const int t_max = n_tiles - 1;
-    load_k(0, 0);
-    load_v(0, 0);
-    load_k(1, 1);
-    load_k(2 < t_max ? 2 : t_max, 2);
-    load_v(1, 1);
-    wait_lds_dma();
-    __syncthreads();
-    qk(0, s_a);
-    row_max_and_rescale(s_a);
-    __syncthreads();  // every wave is done with K slot 0 before step 0 overwrites it
-    const int n_steps = n_tiles / 2;
-    int J = 0;
-    for (; J + 2 < n_steps; J += 2) {
-      step2(integral_constant<int, 0>{}, integral_constant<bool, false>{}, J, s_a, s_b);
-      step2(integral_constant<int, 1>{}, integral_constant<bool, false>{}, J + 1, s_a, s_b);
-    }
-    if (J + 2 == n_steps) {
-      step2(integral_constant<int, 0>{}, integral_constant<bool, false>{}, J, s_a, s_b);
-      step2(integral_constant<int, 1>{}, integral_constant<bool, true>{}, J + 1, s_a, s_b);
-    } else {
-      step2(integral_constant<int, 0>{}, integral_constant<bool, true>{}, J, s_a, s_b);
-    }
+  load_k(0, 0);
+  load_v(0, 0);
+  load_k(n_tiles > 1 ? 1 : 0, 1);
+  wait_lds_dma();
+  __syncthreads();
+  qk(0, s_a);
+  rebase(s_a);
+  __syncthreads();  // every wave is done with K stage 0 before step 0 overwrites it
+  int j = 0;
+  for (; j + 2 < n_tiles; j += 2) {
+    step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
+    step(integral_constant<int, 1>{}, integral_constant<bool, true>{}, j + 1, s_b, s_a);
+  }
+  if (j + 2 == n_tiles) {
+    step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
+    step(integral_constant<int, 1>{}, integral_constant<bool, false>{}, j + 1, s_b, s_a);
   } else {
-    load_k(0, 0);
-    load_v(0, 0);
-    load_k(n_tiles > 1 ? 1 : 0, 1);
-    wait_lds_dma();
-    __syncthreads();
-    qk(0, s_a);
-    row_max_and_rescale(s_a);
-    __syncthreads();  // every wave is done with K stage 0 before step 0 overwrites it
-    int j = 0;
-    for (; j + 2 < n_tiles; j += 2) {
-      step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
-      step(integral_constant<int, 1>{}, integral_constant<bool, true>{}, j + 1, s_b, s_a);
-    }
-    if (j + 2 == n_tiles) {
-      step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
-      step(integral_constant<int, 1>{}, integral_constant<bool, false>{}, j + 1, s_b, s_a);
-    } else {
-      step(integral_constant<int, 0>{}, integral_constant<bool, false>{}, j, s_a, s_b);
-    }
+    step(integral_constant<int, 0>{}, integral_constant<bool, false>{}, j, s_a, s_b);
   }
 
   // ---- epilogue: O = out_scale * O / l (online_softmax.h:59-85), fp16, [B,S,H,D].  A lane holds 4 consecutive d of
@@ -394,12 +305,8 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   float l_tot[QB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    if constexpr (MFMA_SUM) {
-      l_tot[qb] = l_acc[qb][0];
-    } else {
-      l_tot[qb] = l_run[qb] + __shfl_xor(l_run[qb], 16, 64);
-      l_tot[qb] += __shfl_xor(l_tot[qb], 32, 64);
-    }
+    l_tot[qb] = l_run[qb] + __shfl_xor(l_run[qb], 16, 64);
+    l_tot[qb] += __shfl_xor(l_tot[qb], 32, 64);
   }
   {
     char *ot = smem + wave * (32 * C::O_PITCH);
@@ -427,7 +334,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
       *(int4v *)(Op + (int64_t)(q0 + row) * ld + ochunk * 8) = val;
     }
   }
-  if (a.row_max || a.row_sum) {
+  if (want_taps) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       float m_true = fmaxf(m_lane[qb], __shfl_xor(m_lane[qb], 16, 64));

@@ -36,3 +36,14 @@ def subset_pairs(B, H, seed=7):
 
 def max_abs(a, b):
     return float(np.max(np.abs(np.asarray(a, np.float32) - np.asarray(b, np.float32))))
+
+
+def climbing_keys(k, ramp=8.0, spike=40.0):
+    """K [B,Skv,H,D] with key n scaled by 1 + (ramp-1) n/(Skv-1), and one key three quarters along scaled by `spike`
+    on top: the scores grow along the key axis, so the running softmax reference point has to move again and again
+    (online_softmax.h:123-165), by more than the fp16 range (and, for the rows the spike key favours, more than the
+    fp32 range of exp2) in one step."""
+    skv = k.shape[1]
+    w = 1.0 + (ramp - 1.0) * np.arange(skv, dtype=np.float32) / max(skv - 1, 1)
+    w[(3 * skv) // 4 + 3 if skv > 4 else skv - 1] *= spike
+    return k * w[None, :, None, None]

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import oracle
-from _util import ERRPCT_FP16, TOL_FP16, max_abs, pkg, subset_pairs, to_dev
+from _util import ERRPCT_FP16, TOL_FP16, climbing_keys, max_abs, pkg, subset_pairs, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -18,10 +18,12 @@ def _run(q, k, v, **kw):
     return o.float().cpu().numpy(), (q16.astype(np.float32), k16.astype(np.float32), v16.astype(np.float32))
 
 
-def _check_full(B, S, H, D, kind="gaussian", seqlen_kv=None, scale=None):
+def _check_full(B, S, H, D, kind="gaussian", seqlen_kv=None, scale=None, climb=False):
     q, k, v = pkg.testbed.qkv(B, S, H, D, kind=kind, seqlen_kv=seqlen_kv)
     if kind != "gaussian":
         q, k = q / 8, k / 8  # keep scores moderate
+    if climb:
+        k, v = climbing_keys(k), v / 4
     got, (qf, kf, vf) = _run(q, k, v, softmax_scale=scale)
     ref = oracle.attention_f32(qf, kf, vf, alpha0=scale)["O"]
     err = max_abs(got, ref)
@@ -52,6 +54,12 @@ def test_shortest_and_odd_key_tile_counts(B, S, H, D, Skv):
     # one key tile (the pipeline is prologue + last step only), an odd number of tiles (the loop's other tail), and
     # the smallest problem the tiles allow: one workgroup, one (batch, head)
     _check_full(B, S, H, D, seqlen_kv=Skv)
+
+
+@pytest.mark.parametrize("B,S,H,D,Skv", [(1, 256, 2, 64, 512), (2, 256, 2, 128, 384), (1, 128, 2, 256, 256), (1, 128, 1, 128, 64)])
+def test_scores_that_climb_along_the_keys_move_the_reference_point(B, S, H, D, Skv):
+    # the deferred rescale's slow path, many times per row; single-tile case: the reference point is only set
+    _check_full(B, S, H, D, seqlen_kv=Skv, climb=True)
 
 
 def test_integer_valued_inputs():
@@ -143,8 +151,10 @@ def test_invariants_on_device():
     assert max_abs(o.float().cpu().numpy(), base) == 0.0
 
 
-def _subset_check(B, S, H, D):
+def _subset_check(B, S, H, D, climb=False):
     q, k, v = pkg.testbed.qkv(B, S, H, D)
+    if climb:
+        k, v = climbing_keys(k), v / 4
     got, (qf, kf, vf) = _run(q, k, v)
     pairs = subset_pairs(B, H)
     ref = oracle.attention_f32(qf, kf, vf, bh_pairs=pairs)["O"]
@@ -162,6 +172,13 @@ def _subset_check(B, S, H, D):
 def test_config2_headline_shape_subset_check():
     # benchmark configuration 2: B=8 H=16 S=2048 D=128; four full (b,h) slices + every 61st row of every head
     _subset_check(8, 2048, 16, 128)
+
+
+def test_headline_shapes_with_climbing_scores():
+    # the kernels big problems get (256- and 128-row tiles on 16x16x32 MFMAs), on keys that keep moving the softmax
+    # reference point
+    _subset_check(8, 2048, 16, 128, climb=True)
+    _subset_check(4, 2048, 16, 64, climb=True)
 
 
 def test_config3_long_sequence_large_head_subset_check():

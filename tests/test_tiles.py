@@ -12,7 +12,7 @@ from _util import ERRPCT_FP16, ERRPCT_FP8, ROOT, TOL_FP16, TOL_FP8, pkg
 
 # tile wish -> cases (mode:B,S,H,D) that have an instantiation of exactly that tile
 CASES = {
-    "128x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f8:1,2048,2,64", "f8:1,2048,2,128", "f8:1,2048,1,256",
+    "128x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f16climb:1,256,2,128,384", "f8:1,2048,2,64", "f8:1,2048,2,128", "f8:1,2048,1,256",
                "hyb:1,512,2,64", "hyb:1,512,2,128"],
     "256x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f8:1,2048,2,128", "hyb:1,512,2,128"],
     "128x128": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,384,2,128", "f8:1,2048,2,64", "f8:1,2048,2,128",
@@ -20,8 +20,9 @@ CASES = {
     "256x128": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128,384", "f8:1,2048,2,128", "hyb:1,512,2,128"],
     "128x32": ["f16:1,256,2,256", "hyb:1,256,2,256"],
     # the fp16 builds on 16x16x32 MFMAs
-    "128x64/16": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:2,384,3,128,192", "f16:1,256,2,64,64"],
-    "256x64/16": ["f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f16:2,256,1,128,64"],
+    "128x64/16": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:2,384,3,128,192", "f16:1,256,2,64,64", "f16climb:1,256,2,64,512",
+                  "f16climb:1,384,2,128", "f16climb:1,128,1,128,64"],
+    "256x64/16": ["f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f16:2,256,1,128,64", "f16climb:1,512,2,128,448"],
 }
 
 
@@ -80,8 +81,9 @@ def test_forced_tiles_match_the_oracle(wish):
         assert (row["block_m"], row["block_n"]) == (bm, bn), row     # the wished tile really ran
         if row["case"].startswith("f16"):
             assert row["mfma"] == int(mfma or 32), row               # ... on the wished MFMA shape
-            # row-max tap: exact fp32 products, so only summation order separates it from the oracle; row-sum tap:
-            # the kernel adds the weights as rounded to fp16 (2^-11 each, unbiased), the oracle the fp32 values
+            # row-max tap (relative to the largest row max): exact fp32 products, so only summation order separates
+            # it from the oracle; row-sum tap (relative): the kernel adds the weights as rounded to fp16 (2^-11 each,
+            # unbiased), the oracle the fp32 values
             assert row["taps"][0] <= 2e-5 and row["taps"][1] <= 3e-4, row
         fp8 = row["case"].startswith("f8")
         assert not row["nan"] and row["max_abs"] <= (TOL_FP8 if fp8 else TOL_FP16), row

@@ -2,7 +2,8 @@
 the tile wish CFK_FMHA_TILE, read once per process by the library -- and prints one JSON line per case with the
 tile the library planned and the errors against the CPU oracle.
 
-usage: tile_case.py mode:B,S,H,D[,Skv] ...      mode = f16 | f8 | hyb
+usage: tile_case.py mode:B,S,H,D[,Skv] ...      mode = f16 | f8 | hyb, with the suffix `climb` for keys whose scores
+climb along the key axis (tests/_util.py: climbing_keys)
 """
 import json
 import sys
@@ -10,7 +11,7 @@ import sys
 import numpy as np
 
 import oracle
-from _util import max_abs, pkg, to_dev
+from _util import climbing_keys, max_abs, pkg, to_dev
 
 
 def run_case(spec):
@@ -20,6 +21,8 @@ def run_case(spec):
     B, S, H, D = vals[:4]
     Skv = vals[4] if len(vals) > 4 else S
     q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=Skv)
+    if mode.endswith("climb"):
+        mode, k, v = mode[:-5], climbing_keys(k), v / 4
     f = pkg.fmha
     mfma = 32
     if mode == "f16":
@@ -60,7 +63,8 @@ def run_case(spec):
         m_ref, inv_ref = st["row_max"], st["inv_sum"]
         ok = ~np.isnan(m_ref)
         mi = rm.cpu().numpy() / oracle.LOG2E
-        taps = [float(np.abs(mi[ok] - m_ref[ok]).max()), float(np.abs(1.0 / rs.cpu().numpy()[ok] / inv_ref[ok] - 1.0).max())]
+        taps = [float(np.abs(mi[ok] - m_ref[ok]).max() / max(1.0, np.abs(m_ref[ok]).max())),
+                float(np.abs(1.0 / rs.cpu().numpy()[ok] / inv_ref[ok] - 1.0).max())]
     return dict(taps=taps, case=spec, block_m=plan[0], block_n=plan[1], mfma=mfma, lds_bytes=plan[2], checked=int(sel.sum()),
                 max_abs=max_abs(got[sel], ref[sel]), err_pct=pct, nan=bool(np.isnan(got).any()))
 
