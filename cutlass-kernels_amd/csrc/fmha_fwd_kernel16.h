@@ -94,13 +94,13 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   }
   const uint32_t lds_base = (uint32_t)(uintptr_t)LDS_PTR(char, smem);
   const uint32_t lds_wave = lds_base + wave * 1024;  // this wave's 1 KB share of every copy group
-  auto load_k = [&](int jt, int stage) {
+  auto load_k = [&](int jt, int stage) __attribute__((always_inline)) {
     const char *gt = Kp + (size_t)jt * ((size_t)BN * k_ld);
 #pragma unroll
     for (int i = 0; i < C::K_IPW; ++i)
       lds_dma16(gt, goff_k[i], lds_wave, C::K_ST0 + stage * C::K_TILE + i * C::NWAVES * 1024);
   };
-  auto load_v = [&](int jt, int stage) {
+  auto load_v = [&](int jt, int stage) __attribute__((always_inline)) {
     const char *gt = Vp + (size_t)jt * ((size_t)BN * v_ld);
 #pragma unroll
     for (int i = 0; i < C::V_IPW; ++i)
@@ -151,7 +151,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   const bool want_taps = a.row_max != nullptr || a.row_sum != nullptr;
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
   // S^T = K . Q^T for the K tile in LDS slot `stage`
-  auto qk = [&](int stage, f32x4 (&sacc)[KB][QB]) {
+  auto qk = [&](int stage, f32x4 (&sacc)[KB][QB]) __attribute__((always_inline)) {
     const uint32_t kt = stage * C::K_TILE;
 #pragma unroll
     for (int s = 0; s < KS; ++s)
@@ -164,7 +164,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
       }
   };
   // this lane's max over its quarter of the keys of query block qb: a chain of three-operand maxima
-  auto lane_max = [&](const f32x4 (&sacc)[KB][QB], int qb) -> float {
+  auto lane_max = [&](const f32x4 (&sacc)[KB][QB], int qb) __attribute__((always_inline)) -> float {
     float mx = __builtin_fmaxf(sacc[0][qb][0], sacc[0][qb][1]);
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
@@ -174,7 +174,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   };
   // Move the reference point of every query up to the row max of `sacc` (if that is above it) and re-base O and l
   // (online_softmax.h:123-165); for the first tile the old reference point is -inf and O and l are zero.
-  auto rebase = [&](const f32x4 (&sacc)[KB][QB]) {
+  auto rebase = [&](const f32x4 (&sacc)[KB][QB]) __attribute__((always_inline)) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       const float mx = lane_max(sacc, qb);
@@ -190,7 +190,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   };
   // P = exp2(c*S - m_ref), cast to fp16 in the B-operand register order of the second GEMM, and the tile's row sums of
   // P as rounded (the weights the second GEMM applies), in fp32
-  auto exp_and_sum = [&](const f32x4 (&sacc)[KB][QB], half8 (&pb)[QB][PS], float (&rsum)[QB]) {
+  auto exp_and_sum = [&](const f32x4 (&sacc)[KB][QB], half8 (&pb)[QB][PS], float (&rsum)[QB]) __attribute__((always_inline)) {
     const half2v one2 = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -216,7 +216,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
   // the (wave-uniform, rare) slow path: the scores are gone by then (the exponentials overwrote them; keeping them
   // would cost 32 registers), so it recomputes them with K fragments fetched straight from global memory, moves the
   // reference point up to their row max and takes the exponentials again.
-  auto softmax_tile = [&](int jt, const f32x4 (&sacc)[KB][QB], half8 (&pb)[QB][PS]) {
+  auto softmax_tile = [&](int jt, const f32x4 (&sacc)[KB][QB], half8 (&pb)[QB][PS]) __attribute__((always_inline)) {
     if (want_taps) {
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) m_lane[qb] = __builtin_fmaxf(m_lane[qb], lane_max(sacc, qb));
@@ -245,7 +245,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
     for (int qb = 0; qb < QB; ++qb) l_run[qb] += rsum[qb];
   };
   // O^T += V^T . P^T for the V tile at LDS byte offset vt
-  auto pv = [&](uint32_t vt, const half8 (&pb)[QB][PS]) {
+  auto pv = [&](uint32_t vt, const half8 (&pb)[QB][PS]) __attribute__((always_inline)) {
 #pragma unroll
     for (int ps = 0; ps < PS; ++ps)
 #pragma unroll
@@ -264,7 +264,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
 
   // One pipeline step for tile j (parity P = j & 1), as in fmha_fwd_kernel.h: on entry s_cur = S_j is finished, K_{j+1}
   // sits in K stage P^1 and V_j in V stage P.
-  auto step = [&](auto parity, auto has_next, int j, f32x4 (&s_cur)[KB][QB], f32x4 (&s_nxt)[KB][QB]) {
+  auto step = [&](auto parity, auto has_next, int j, f32x4 (&s_cur)[KB][QB], f32x4 (&s_nxt)[KB][QB]) __attribute__((always_inline)) {
     constexpr int P = decltype(parity)::value;
     constexpr bool HAS_NEXT = decltype(has_next)::value;
     load_k(j + 2 < n_tiles ? j + 2 : n_tiles - 1, P);
