@@ -228,7 +228,11 @@ fmha_fwd_kernel16(const FmhaArgs a) {
     for (int qb = 0; qb < QB; ++qb) over = over || !(rsum[qb] < sum_cap);
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(over) != 0, 0)) {
       f32x4 sr[KB][QB];
-      const char *kt = Kp + (size_t)jt * ((size_t)BN * k_ld) + (size_t)c * k_ld + 16 * g;
+      // (the empty statement keeps the address arithmetic of this path inside it: hoisted out of the loop it would
+      // occupy ten registers for all of the kernel)
+      int cc = c, gg = g;
+      asm volatile("" : "+v"(cc), "+v"(gg));
+      const char *kt = Kp + (size_t)jt * ((size_t)BN * k_ld) + (size_t)cc * k_ld + 16 * gg;
 #pragma unroll
       for (int s = 0; s < KS; ++s)
 #pragma unroll
