@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import oracle
-from _util import ERRPCT_FP8, TOL_FP8, max_abs, pkg, subset_pairs, to_dev
+from _util import ERRPCT_FP8, TOL_FP8, climbing_keys, max_abs, pkg, subset_pairs, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -77,6 +77,35 @@ def test_shapes_per_tensor_scales(B, S, H, D):
 @pytest.mark.parametrize("B,S,H,D,Skv", [(1, 128, 1, 64, 64), (1, 128, 1, 128, 64), (2, 256, 2, 128, 192), (1, 128, 2, 256, 64)])
 def test_shortest_and_odd_key_tile_counts(B, S, H, D, Skv):
     _check_full(B, S, H, D, seqlen_kv=Skv)
+
+
+@pytest.mark.parametrize("mode", ["fp8", "hybrid"])
+@pytest.mark.parametrize("B,S,H,D,Skv", [(1, 256, 2, 128, 512), (1, 128, 2, 64, 384), (1, 128, 1, 256, 256), (1, 128, 1, 128, 64),
+                                         (2, 2048, 8, 128, 2048)])
+def test_scores_that_climb_along_the_keys_move_the_reference_point(mode, B, S, H, D, Skv):
+    # the deferred rescale's slow path, many times per row (e4m3 P has two binades of head-room above the row max of
+    # the moment, so here almost every tile takes it); the last shape gets the 256-row tile with two sub-tiles per barrier
+    import torch
+    from _util import TOL_FP16
+    q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=Skv)
+    k, v = climbing_keys(k, ramp=4.0, spike=8.0), v / 4
+    (qc, qs, qf), (kc, ks, kf) = _quant(q), _quant(k)
+    if mode == "fp8":
+        vc, vs, vf = _quant(v)
+        o = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(vc), q_descale=qs, k_descale=ks, v_descale=vs)
+    else:
+        v16 = v.astype(np.float16)
+        vf = v16.astype(np.float32)
+        o = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(v16), q_descale=qs, k_descale=ks)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    pairs = sorted({(0, 0), (B - 1, H - 1)})
+    ref = oracle.attention_f32(qf, kf, vf, bh_pairs=pairs)["O"]
+    sel = ~np.isnan(ref)
+    err = max_abs(got[sel], ref[sel])
+    print(f"{mode} climbing B={B} S={S}/{Skv} H={H} D={D}: max-abs {err:.3e}")
+    assert not np.isnan(got).any()
+    assert err <= (TOL_FP8 if mode == "fp8" else TOL_FP16), err
 
 
 def test_reference_mode_unit_scales():
