@@ -21,12 +21,16 @@ using C128_128x128 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 2>;
 using C128_256x128 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 2>;
 using C256_128x32 = FmhaCfg<256, 32, 4, 1, false, false>;
 using C256_128x32P = FmhaCfg<256, 32, 4, 1, false, false, false, false, 1, 4>;  // key length a multiple of 128
-// The builds on 16x16x32 MFMAs, the automatic choice for big problems at head dims 64 and 128 (+3..5 % on N(0,1)
-// data).  Not built: the K fragment prefetch and the two-tile step (registers spill or nothing is gained), 256 rows
-// at head dim 64 (880 against 919 TFLOP/s for 128 rows), head dim 256 (929 against 932 for the 32x32 build).
+// The builds on 16x16x32 MFMAs, the automatic choice for big problems at head dims 64 and 128 (+6..10 % on N(0,1)
+// data).  Head dim 128: two key tiles per barrier when the key length allows (+1..2 %: 1145-1157 against 1134
+// TFLOP/s on B=8 H=16 S=2048).  Not built: the K fragment prefetch (registers spill), at head dim 64 256 rows (880
+// against 919 TFLOP/s for 128 rows) and two tiles per barrier (950 against 1030: the LDS then holds two workgroups
+// per CU, not three), head dim 256 (929 against 932 for the 32x32 build).
 using N64_128x64 = FmhaCfg<64, 64, 4, 3, false, false, false, false, 1, 0, true>;
 using N128_128x64 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 1, 0, true>;
 using N128_256x64 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 1, 0, true>;
+using N128_256x128 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 2, 0, true>;
+using N128_128x128 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 2, 0, true>;
 
 // builds that also write the score tap (debug): 128-row tile only
 using C64Tap = FmhaCfg<64, 64, 4, 2, false, false, false, true>;
@@ -34,7 +38,7 @@ using C128Tap = FmhaCfg<128, 64, 4, 2, false, false, false, true>;
 using C256Tap = FmhaCfg<256, 32, 4, 1, false, false, false, true>;
 
 using All64 = CfgList<C64_128x64, N64_128x64, C64_256x64, C64_128x128, C64_256x128>;
-using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128>;
+using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128, N128_128x128, N128_256x128>;
 // head dim 256: 64-key tiles and two 32-key tiles per barrier both spill registers inside the loop (572 against 940
 // TFLOP/s on B=2 H=8 S=8192): not built
 using All256 = CfgList<C256_128x32P, C256_128x32>;
@@ -51,7 +55,7 @@ bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
   }
   switch (head_dim) {
     case 64: select_tile<All64, CfgList<N64_128x64, C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
-    case 128: select_tile<All128, CfgList<N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
+    case 128: select_tile<All128, CfgList<N128_256x128, N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
     case 256: select_tile<All256, All256, C256_128x32>(sq, skv, bh, f); return true;
     default: return false;
   }

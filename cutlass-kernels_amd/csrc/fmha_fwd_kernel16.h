@@ -146,7 +146,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) l_run[qb] = 0.f;
 
-  static_assert(C::KPRE == 0 && C::SUB == 1, "one key tile per barrier, no K fragment prefetch in this kernel");
+  static_assert(C::KPRE == 0, "no K fragment prefetch in this kernel");
   const float sum_cap = __builtin_amdgcn_exp2f(kTau);
   const bool want_taps = a.row_max != nullptr || a.row_sum != nullptr;
   const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -281,26 +281,78 @@ fmha_fwd_kernel16(const FmhaArgs a) {
     __syncthreads();
   };
 
+  // Two key tiles per barrier (SUB = 2), slot bookkeeping as in fmha_fwd_kernel.h: tile t of K and of V lives in slot
+  // t % 4; step J covers tiles 2J and 2J+1 and refills the slots last read by step J-1.
+  auto step2 = [&](auto parity, auto last, int J, f32x4 (&s_a)[KB][QB], f32x4 (&s_b)[KB][QB]) __attribute__((always_inline)) {
+    constexpr int P = decltype(parity)::value;
+    constexpr bool LAST = decltype(last)::value;
+    const int t0 = 2 * J, t_max = n_tiles - 1;
+    load_k(t0 + 3 < t_max ? t0 + 3 : t_max, (2 * P + 3) % 4);
+    load_k(t0 + 4 < t_max ? t0 + 4 : t_max, (2 * P) % 4);
+    {
+      half8 pb[QB][PS];
+      qk((2 * P + 1) % 4, s_b);
+      softmax_tile(t0, s_a, pb);
+      pv(((2 * P) % 4) * C::V_TILE, pb);
+    }
+    load_v(t0 + 2 < t_max ? t0 + 2 : t_max, (2 * P + 2) % 4);
+    load_v(t0 + 3 < t_max ? t0 + 3 : t_max, (2 * P + 3) % 4);
+    {
+      half8 pb[QB][PS];
+      if (!LAST) qk((2 * P + 2) % 4, s_a);
+      softmax_tile(t0 + 1, s_b, pb);
+      pv(((2 * P + 1) % 4) * C::V_TILE, pb);
+    }
+    wait_lds_dma();
+    __syncthreads();
+  };
+
   using std::integral_constant;
   f32x4 s_a[KB][QB], s_b[KB][QB];
-  load_k(0, 0);
-  load_v(0, 0);
-  load_k(n_tiles > 1 ? 1 : 0, 1);
-  wait_lds_dma();
-  __syncthreads();
-  qk(0, s_a);
-  rebase(s_a);
-  __syncthreads();  // every wave is done with K stage 0 before step 0 overwrites it
-  int j = 0;
-  for (; j + 2 < n_tiles; j += 2) {
-    step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
-    step(integral_constant<int, 1>{}, integral_constant<bool, true>{}, j + 1, s_b, s_a);
-  }
-  if (j + 2 == n_tiles) {
-    step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
-    step(integral_constant<int, 1>{}, integral_constant<bool, false>{}, j + 1, s_b, s_a);
+  if constexpr (C::SUB == 2) {
+    const int t_max = n_tiles - 1;
+    load_k(0, 0);
+    load_v(0, 0);
+    load_k(1, 1);
+    load_k(2 < t_max ? 2 : t_max, 2);
+    load_v(1, 1);
+    wait_lds_dma();
+    __syncthreads();
+    qk(0, s_a);
+    rebase(s_a);
+    __syncthreads();  // every wave is done with K slot 0 before step 0 overwrites it
+    const int n_steps = n_tiles / 2;
+    int J = 0;
+    for (; J + 2 < n_steps; J += 2) {
+      step2(integral_constant<int, 0>{}, integral_constant<bool, false>{}, J, s_a, s_b);
+      step2(integral_constant<int, 1>{}, integral_constant<bool, false>{}, J + 1, s_a, s_b);
+    }
+    if (J + 2 == n_steps) {
+      step2(integral_constant<int, 0>{}, integral_constant<bool, false>{}, J, s_a, s_b);
+      step2(integral_constant<int, 1>{}, integral_constant<bool, true>{}, J + 1, s_a, s_b);
+    } else {
+      step2(integral_constant<int, 0>{}, integral_constant<bool, true>{}, J, s_a, s_b);
+    }
   } else {
-    step(integral_constant<int, 0>{}, integral_constant<bool, false>{}, j, s_a, s_b);
+    load_k(0, 0);
+    load_v(0, 0);
+    load_k(n_tiles > 1 ? 1 : 0, 1);
+    wait_lds_dma();
+    __syncthreads();
+    qk(0, s_a);
+    rebase(s_a);
+    __syncthreads();  // every wave is done with K stage 0 before step 0 overwrites it
+    int j = 0;
+    for (; j + 2 < n_tiles; j += 2) {
+      step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
+      step(integral_constant<int, 1>{}, integral_constant<bool, true>{}, j + 1, s_b, s_a);
+    }
+    if (j + 2 == n_tiles) {
+      step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, j, s_a, s_b);
+      step(integral_constant<int, 1>{}, integral_constant<bool, false>{}, j + 1, s_b, s_a);
+    } else {
+      step(integral_constant<int, 0>{}, integral_constant<bool, false>{}, j, s_a, s_b);
+    }
   }
 
   // ---- epilogue: O = out_scale * O / l (online_softmax.h:59-85), fp16, [B,S,H,D].  A lane holds 4 consecutive d of

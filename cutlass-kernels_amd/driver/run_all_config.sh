@@ -14,13 +14,13 @@ HERE="$(cd "$(dirname "$0")" && pwd)"
 BATCH=${BATCH:-4}; SEQ=${SEQ:-4096}; DIM=${DIM:-2048}; ITERS=${ITERS:-1000}
 MODES=( fp16 fp8 fp8-bdhs hybrid )
 HEADSIZES=( 64 128 256 )
-TILES=( 128x64 256x64 128x128 256x128 128x64/16 256x64/16 )
+TILES=( 128x64 256x64 128x128 256x128 128x64/16 256x64/16 128x128/16 256x128/16 )
 MODE=$1
 STATUS=0
 # the tile shapes that exist per mode and head size (the others would silently run the default tile)
 has_tile() {  # mode head tile
   case "$1:$2" in
-    fp16:64) [[ $3 != 128x32 && $3 != 256x64/16 ]] ;;
+    fp16:64) [[ $3 != 128x32 && $3 != 256x64/16 && $3 != *x128/16 ]] ;;
     fp16:128) [[ $3 != 128x32 ]] ;;
     fp16:256|hybrid:256) [[ $3 == 128x32 ]] ;;
     fp8:128) [[ $3 != 128x32 && $3 != */16 ]] ;;

@@ -23,6 +23,8 @@ CASES = {
     "128x64/16": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:2,384,3,128,192", "f16:1,256,2,64,64", "f16climb:1,256,2,64,512",
                   "f16climb:1,384,2,128", "f16climb:1,128,1,128,64"],
     "256x64/16": ["f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f16:2,256,1,128,64", "f16climb:1,512,2,128,448"],
+    "128x128/16": ["f16:1,512,2,128", "f16:2,384,3,128,128", "f16:1,256,2,128,640", "f16climb:1,384,2,128"],
+    "256x128/16": ["f16:1,512,2,128", "f16:1,768,2,128,384", "f16:2,256,1,128,128", "f16climb:1,512,2,128,768"],
 }
 
 
@@ -54,7 +56,10 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     assert shapes("256x64/16") == "16 32 32 32 (256, 64)"      # no 256-row 16x16x32 build at head dim 64
     assert shapes("256x64/32") == "32 32 32 32 (256, 64)"
     assert shapes("128x64") == "32 32 32 32 (128, 64)"
-    assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:2] == (256, 64)   # big problem: automatic choice
+    assert shapes("256x128") == "32 32 32 32 (256, 128)"
+    assert shapes("256x128/16") == "16 32 32 32 (256, 128)"   # two key tiles per barrier on 16x16x32: head dim 128 only
+    assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:2] == (256, 128)  # big problem: automatic choice
+    assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 1984, 128)[:2] == (256, 64)   # ... key length not a multiple of 128
     # ... on 16x16x32 MFMAs for fp16 at head dims 64 and 128; small problems, head dim 256 and e4m3 stay on 32x32
     assert f.fmha_forward_mfma(f.CFK_FP16, 8, 16, 2048, 2048, 128) == 16
     assert f.fmha_forward_mfma(f.CFK_FP16, 4, 32, 4096, 4096, 64) == 16
@@ -84,7 +89,8 @@ def test_forced_tiles_match_the_oracle(wish):
             # row-max tap (relative to the largest row max): exact fp32 products, so only summation order separates
             # it from the oracle; row-sum tap (relative): the kernel adds the weights as rounded to fp16 (2^-11 each,
             # unbiased), the oracle the fp32 values
-            assert row["taps"][0] <= 2e-5 and row["taps"][1] <= 3e-4, row
+            # (with climbing keys one or two weights carry a row's sum: no averaging, up to 2^-11 = 4.9e-4)
+            assert row["taps"][0] <= 2e-5 and row["taps"][1] <= (5e-4 if "climb" in row["case"] else 3e-4), row
         fp8 = row["case"].startswith("f8")
         assert not row["nan"] and row["max_abs"] <= (TOL_FP8 if fp8 else TOL_FP16), row
         assert row["err_pct"] <= (ERRPCT_FP8 if fp8 else ERRPCT_FP16), row
