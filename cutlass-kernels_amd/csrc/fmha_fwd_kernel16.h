@@ -1,5 +1,5 @@
 // The fp16 FMHA forward kernel on 16x16x32 MFMAs (v_mfma_f32_16x16x32_f16).  Same algorithm, LDS staging, pipeline
-// (the plain one-tile-per-barrier form) and epilogue as fmha_fwd_kernel.h, which it takes its configuration struct and
+// (one or two key tiles per barrier) and epilogue as fmha_fwd_kernel.h, which it takes its configuration struct and
 // host-side plumbing from; what differs is the MFMA shape, with it every register layout, and how the softmax notices
 // that its reference point has to move: not by a row max per tile but by the row sum it needs anyway (softmax_tile
 // below; 22 VALU instructions per wave and tile less, +3..6 % on N(0,1) data, results bit-identical).
