@@ -509,10 +509,10 @@ fmha_fwd_kernel(const FmhaArgs a) {
     __syncthreads();
   };
 
-  // ---- Two passes over the keys.  The first one takes the row max of the first tile only and then trusts the range
-  // of P: no row max, no comparison, no branch per tile (on N(0,1) data +14 % for e4m3 operands, +28 % at head dim
-  // 256).  A weight that leaves the range of its format turns into infinity (fp16) or NaN (e4m3; v_cvt_pk_fp8_f32 has
-  // no infinity) and from there into a non-finite O and l for that query, which is looked for once, after the loop.
+  // ---- Two passes over the keys (e4m3 P).  The first one takes the row max of the first tile only and then trusts
+  // the range of P: no row max, no comparison, no branch per tile (on N(0,1) data +14 % at head dims 64 and 128).  A
+  // weight that leaves the range of e4m3 turns into NaN (v_cvt_pk_fp8_f32 has no infinity; it does so above 464) and
+  // from there into a non-finite O and l for that query, which is looked for once, after the loop.
   // Only if some row of the workgroup shows it, the keys are walked again with the row max tracked tile by tile, the
   // reference's algorithm (online_softmax.h:123-165).  The taps need the true row max: they go straight to that pass,
   // and so do e4m3 weights on short key sequences (tau = 0: there the row's largest weight has to stay an exact power
@@ -603,7 +603,8 @@ fmha_fwd_kernel(const FmhaArgs a) {
     }
 
   };
-  bool redo = C::TAP_S || a.row_max != nullptr || a.row_sum != nullptr || (PV8 && !(kTau > 0.f));
+  // (fp16 P gains nothing from the first pass -- its row max hides behind the second GEMM's MFMAs -- and skips it.)
+  bool redo = !PV8 || C::TAP_S || a.row_max != nullptr || a.row_sum != nullptr || !(kTau > 0.f);
   if (!redo) {
     pass(integral_constant<bool, false>{});
     const float l_chk = MFMA_SUM ? l_acc[0] : l_run;
