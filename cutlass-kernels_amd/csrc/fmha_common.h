@@ -34,6 +34,11 @@ hipError_t launch_fmha_f16(const FmhaArgs &a, int head_dim, hipStream_t s);     
 hipError_t launch_fmha_fp8(const FmhaArgs &a, int head_dim, hipStream_t s);      // Q,K,V e4m3, P e4m3
 hipError_t launch_fmha_hybrid(const FmhaArgs &a, int head_dim, hipStream_t s);   // Q,K e4m3; P,V fp16
 bool plan_fmha_f16(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *p);
+// fp16 at head dim 256 (without the score tap) lives in a translation unit of its own; launch_fmha_f16 and
+// plan_fmha_f16 forward to these
+hipError_t launch_fmha_f16_d256(const FmhaArgs &a, hipStream_t s);
+void plan_fmha_f16_d256(int sq, int skv, int bh, FmhaPlan *p);
+hipError_t prepare_fmha_f16_d256();
 bool plan_fmha_fp8(int head_dim, int sq, int skv, int bh, int v_layout, bool tap_s, FmhaPlan *p);
 bool plan_fmha_hybrid(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *p);
 // One-time set-up (dynamic-LDS limits) of every instantiation of a family on the current device; launches do it on

@@ -8,8 +8,8 @@ namespace {
 // <head dim, keys per tile, waves, waves per SIMD, e4m3 Q/K, e4m3 P/V, V transposed, score tap, tiles per barrier,
 //  K fragments read ahead of the barrier, 16x16x32 build>.  4 waves = 128 query rows (two workgroups share a CU),
 // 8 waves = 256 rows (one workgroup per CU, half the K/V traffic per query row).  Two waves per SIMD, except head dim
-// 64, whose 128-row tile fits three (the faster choice there), and head dim 256 (Q + O fill half the register file:
-// one).
+// 64, whose 128-row tile fits three (the faster choice there).  Head dim 256 (one wave per SIMD) is built in
+// fmha_fwd_f16_d256.hip, under a machine-scheduler strategy of its own; only its score-tap build is here.
 using C64_128x64 = FmhaCfg<64, 64, 4, 3, false, false>;
 using C64_256x64 = FmhaCfg<64, 64, 8, 2, false, false>;
 using C64_128x128 = FmhaCfg<64, 64, 4, 2, false, false, false, false, 2>;
@@ -19,8 +19,6 @@ using C128_256x64 = FmhaCfg<128, 64, 8, 2, false, false>;
 using C128_256x64P = FmhaCfg<128, 64, 8, 2, false, false, false, false, 1, 4>;  // key length a multiple of 256
 using C128_128x128 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 2>;
 using C128_256x128 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 2>;
-using C256_128x32 = FmhaCfg<256, 32, 4, 1, false, false>;
-using C256_128x32P = FmhaCfg<256, 32, 4, 1, false, false, false, false, 1, 4>;  // key length a multiple of 128
 // The builds on 16x16x32 MFMAs, the automatic choice for big problems at head dims 64 and 128 (+6..10 % on N(0,1)
 // data).  Head dim 128: two key tiles per barrier when the key length allows (+1..2 %: 1145-1157 against 1134
 // TFLOP/s on B=8 H=16 S=2048).  Not built: the K fragment prefetch (registers spill), at head dim 64 256 rows (880
@@ -39,9 +37,6 @@ using C256Tap = FmhaCfg<256, 32, 4, 1, false, false, false, true>;
 
 using All64 = CfgList<C64_128x64, N64_128x64, C64_256x64, C64_128x128, C64_256x128>;
 using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128, N128_128x128, N128_256x128>;
-// head dim 256: 64-key tiles and two 32-key tiles per barrier both spill registers inside the loop (572 against 940
-// TFLOP/s on B=2 H=8 S=8192): not built
-using All256 = CfgList<C256_128x32P, C256_128x32>;
 
 template <class F>
 bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
@@ -56,7 +51,6 @@ bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
   switch (head_dim) {
     case 64: select_tile<All64, CfgList<N64_128x64, C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
     case 128: select_tile<All128, CfgList<N128_256x128, N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
-    case 256: select_tile<All256, All256, C256_128x32>(sq, skv, bh, f); return true;
     default: return false;
   }
 }
@@ -64,10 +58,12 @@ bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
 }  // namespace
 
 bool plan_fmha_f16(int head_dim, int sq, int skv, int bh, bool tap_s, FmhaPlan *p) {
+  if (head_dim == 256 && !tap_s) { plan_fmha_f16_d256(sq, skv, bh, p); return true; }
   return dispatch(head_dim, sq, skv, bh, tap_s, [&](auto cfg) { fill_fmha_plan<decltype(cfg)>(sq, bh, p); });
 }
 
 hipError_t launch_fmha_f16(const FmhaArgs &a, int head_dim, hipStream_t s) {
+  if (head_dim == 256 && !a.s_tap) return launch_fmha_f16_d256(a, s);
   hipError_t e = hipErrorInvalidValue;
   dispatch(head_dim, a.Sq, a.Skv, a.B * a.H, a.s_tap != nullptr, [&](auto cfg) { e = launch_fmha_cfg<decltype(cfg)>(a, s); });
   return e;
@@ -76,7 +72,7 @@ hipError_t launch_fmha_f16(const FmhaArgs &a, int head_dim, hipStream_t s) {
 hipError_t prepare_fmha_f16() {
   hipError_t e = prepare_all(All64{});
   if (e == hipSuccess) e = prepare_all(All128{});
-  if (e == hipSuccess) e = prepare_all(All256{});
+  if (e == hipSuccess) e = prepare_fmha_f16_d256();
   if (e == hipSuccess) e = prepare_all(CfgList<C64Tap, C128Tap, C256Tap>{});
   return e;
 }

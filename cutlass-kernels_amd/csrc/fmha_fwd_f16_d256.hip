@@ -1,0 +1,39 @@
+// FMHA forward, fp16 operands, head dim 256: tile shapes and dispatch.  A translation unit of its own because these
+// kernels run one wave per SIMD (Q and O fill half the register file) and are built with another machine-scheduler
+// strategy than the rest of the library (Makefile: iterative-ilp).  With a single wave nothing but the wave's own
+// instruction order hides LDS and MFMA latency, and the order that strategy finds is the faster one: 994-1001 against
+// 928 TFLOP/s on B=2 H=8 S=8192 with N(0,1) tensors, 1206 against 1024 with constant tensors.  Every kernel with two or
+// three waves per SIMD loses under it (registers spill), so it is not a library-wide flag.
+#include "fmha_fwd_kernel.h"
+
+namespace cfk {
+namespace {
+
+// <head dim, keys per tile, waves, waves per SIMD, e4m3 Q/K, e4m3 P/V, V transposed, score tap, tiles per barrier,
+//  K fragments read ahead of the barrier>
+using C256_128x32 = FmhaCfg<256, 32, 4, 1, false, false>;
+using C256_128x32P = FmhaCfg<256, 32, 4, 1, false, false, false, false, 1, 4>;  // key length a multiple of 128
+// 64-key tiles and two 32-key tiles per barrier both spill registers inside the loop (572 against 940 TFLOP/s on
+// B=2 H=8 S=8192): not built
+using All256 = CfgList<C256_128x32P, C256_128x32>;
+
+template <class F>
+void dispatch(int sq, int skv, int bh, F &&f) {
+  select_tile<All256, All256, C256_128x32>(sq, skv, bh, f);
+}
+
+}  // namespace
+
+void plan_fmha_f16_d256(int sq, int skv, int bh, FmhaPlan *p) {
+  dispatch(sq, skv, bh, [&](auto cfg) { fill_fmha_plan<decltype(cfg)>(sq, bh, p); });
+}
+
+hipError_t launch_fmha_f16_d256(const FmhaArgs &a, hipStream_t s) {
+  hipError_t e = hipErrorInvalidValue;
+  dispatch(a.Sq, a.Skv, a.B * a.H, [&](auto cfg) { e = launch_fmha_cfg<decltype(cfg)>(a, s); });
+  return e;
+}
+
+hipError_t prepare_fmha_f16_d256() { return prepare_all(All256{}); }
+
+}  // namespace cfk
