@@ -22,7 +22,8 @@ has_tile() {  # mode head tile
   case "$1:$2" in
     fp16:64) [[ $3 != 128x32 && $3 != 256x64/16 && $3 != *x128/16 ]] ;;
     fp16:128) [[ $3 != 128x32 ]] ;;
-    fp16:256|hybrid:256) [[ $3 == 128x32 ]] ;;
+    fp16:256) [[ $3 == 128x32 || $3 == 128x64 ]] ;;
+    hybrid:256) [[ $3 == 128x32 ]] ;;
     fp8:128) [[ $3 != 128x32 && $3 != */16 ]] ;;
     fp8:64|fp8:256) [[ $3 == 128x64 || $3 == 128x128 ]] ;;
     fp8-bdhs:*) [[ $3 == 128x64 ]] ;;

@@ -100,7 +100,7 @@ def test_sweep_script_verify_all_on_a_reduced_problem():
     r = subprocess.run(["bash", script, "verify-all"], env=env, capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout[-4000:] + r.stderr[-2000:]
     blocks = r.stdout.split("CONFIG ")[1:]
-    assert len(blocks) == 31, len(blocks)
+    assert len(blocks) == 32, len(blocks)
     seen = set()
     for blk in blocks:
         head_line = blk.splitlines()[0]
@@ -113,7 +113,7 @@ def test_sweep_script_verify_all_on_a_reduced_problem():
             assert line in blk, (head_line, blk)
         assert "Failed" not in blk
         seen.add((mode, head, tile))
-    assert len(seen) == 31
+    assert len(seen) == 32
     assert {m for m, _, _ in seen} == {"fp16", "fp8", "fp8-bdhs", "hybrid"}
 
 

@@ -13,7 +13,7 @@ from _util import ERRPCT_FP16, ERRPCT_FP8, ROOT, TOL_FP16, TOL_FP8, pkg
 # tile wish -> cases (mode:B,S,H,D) that have an instantiation of exactly that tile
 CASES = {
     "128x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f16climb:1,256,2,128,384", "f8:1,2048,2,64", "f8:1,2048,2,128", "f8:1,2048,1,256",
-               "hyb:1,512,2,64", "hyb:1,512,2,128"],
+               "hyb:1,512,2,64", "hyb:1,512,2,128", "f16:1,256,2,256", "f16climb:1,256,1,256,192"],
     "256x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f8:1,2048,2,128", "hyb:1,512,2,128"],
     "128x128": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,384,2,128", "f8:1,2048,2,64", "f8:1,2048,2,128",
                 "f8:1,2048,1,256", "hyb:1,512,2,64"],
