@@ -81,12 +81,18 @@ def test_shortest_and_odd_key_tile_counts(B, S, H, D, Skv):
 
 @pytest.mark.parametrize("mode", ["fp8", "hybrid"])
 @pytest.mark.parametrize("B,S,H,D,Skv", [(1, 256, 2, 128, 512), (1, 128, 2, 64, 384), (1, 128, 1, 256, 256), (1, 128, 1, 128, 64),
-                                         (2, 2048, 8, 128, 2048)])
+                                         (2, 2048, 32, 128, 2048)])
 def test_scores_that_climb_along_the_keys_move_the_reference_point(mode, B, S, H, D, Skv):
     # the deferred rescale's slow path, many times per row (e4m3 P has two binades of head-room above the row max of
-    # the moment, so here almost every tile takes it); the last shape gets the 256-row tile with two sub-tiles per barrier
+    # the moment, so here almost every tile takes it); with 2048 keys the e4m3 kernel starts in its pass without a row
+    # max per tile, finds non-finite rows and walks the keys again.  The last shape is large enough for the automatic
+    # choice of the 256-row tile (two sub-tiles per barrier for e4m3 P).
     import torch
     from _util import TOL_FP16
+    if B * H * (S // 256) >= 512:
+        f = pkg.fmha
+        plan = f.fmha_forward_plan(f.CFK_FP8_E4M3, B, H, S, Skv, D, v_dtype=f.CFK_FP8_E4M3 if mode == "fp8" else f.CFK_FP16)
+        assert plan[:2] == ((256, 128) if mode == "fp8" else (256, 64)), plan
     q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=Skv)
     k, v = climbing_keys(k, ramp=4.0, spike=8.0), v / 4
     (qc, qs, qf), (kc, ks, kf) = _quant(q), _quant(k)
