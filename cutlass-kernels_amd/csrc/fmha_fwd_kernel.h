@@ -436,6 +436,33 @@ fmha_fwd_kernel(const FmhaArgs a) {
       }
   };
 
+  // e4m3 P: the three parts of a tile's work -- S_{j+1} = K.Q^T, the exponentials of S_j, O += P.V -- are kept apart as
+  // blocks (scheduling fences) instead of being interleaved by the compiler.  The VALU is the busy unit of that kernel
+  // (per key the softmax costs what it costs for fp16 P, the MFMA time is halved); with the blocks apart the two waves
+  // of a SIMD overlap one wave's exponentials with the other's MFMAs: B=4 H=16 S=4096 D=128 2243-2334 against 2198-2269
+  // TFLOP/s on N(0,1) tensors (two boxes), 2798 against 2664 on constant ones; head dim 64 +1.2 %.  One wave per SIMD
+  // (head dim 256) gains most with the exponentials in front of the first GEMM: 2124 against 2050 (+0.8 % in the other
+  // order).  With fp16 P the same fences lose (hybrid -2..-8 %, fp16 -2..-10 %): those kernels keep the compiler's order.
+  constexpr bool FENCED = PV8;
+  constexpr bool EXP_FIRST = PV8 && C::WPE == 1;
+  auto fence = [&]() __attribute__((always_inline)) {
+    if constexpr (FENCED) __builtin_amdgcn_sched_barrier(0);
+  };
+  // qk(next) and the exponentials of the current tile, in the order of the build
+  auto qk_and_exp = [&](auto has_next, int k_stage, f32x16 (&s_nxt)[KB], f32x16 (&s_cur)[KB], PReg (&pb)[PS]) __attribute__((always_inline)) {
+    constexpr bool HAS_NEXT = decltype(has_next)::value;
+    if constexpr (EXP_FIRST) {
+      softmax_exp(s_cur, pb);
+      fence();
+      if (HAS_NEXT) qk(k_stage, s_nxt);
+    } else {
+      if (HAS_NEXT) qk(k_stage, s_nxt);
+      fence();
+      softmax_exp(s_cur, pb);
+    }
+    fence();
+  };
+
   // One pipeline step for tile j (parity P = j & 1).  On entry: s_cur = S_j is finished and its max is folded into
   // m_ref; K_{j+1} sits in K stage P^1 and V_j in V stage P.  HAS_NEXT is false for the last tile only.
   auto step = [&](auto track, auto parity, auto has_next, int j, f32x16 (&s_cur)[KB], f32x16 (&s_nxt)[KB]) __attribute__((always_inline)) {
@@ -447,8 +474,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
     load_k(j + 2 < n_tiles ? j + 2 : n_tiles - 1, P);
     load_v(j + 1 < n_tiles ? j + 1 : n_tiles - 1, P ^ 1);
     PReg pb[PS];
-    if (HAS_NEXT) qk(P ^ 1, s_nxt);
-    softmax_exp(s_cur, pb);
+    qk_and_exp(has_next, P ^ 1, s_nxt, s_cur, pb);
     pv(P * C::V_TILE, pb);
     if (TRACK && HAS_NEXT) row_max_and_rescale(s_nxt, j + 1);
     wait_lds_dma();   // this wave's copies have landed ...
@@ -468,8 +494,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
     load_k(t0 + 4 < t_max ? t0 + 4 : t_max, (2 * P) % 4);
     {
       PReg pb[PS];
-      qk((2 * P + 1) % 4, s_b);
-      softmax_exp(s_a, pb);
+      qk_and_exp(std::true_type{}, (2 * P + 1) % 4, s_b, s_a, pb);
       pv(((2 * P) % 4) * C::V_TILE, pb);
       if (TRACK) row_max_and_rescale(s_b, t0 + 1);
     }
@@ -477,8 +502,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
     load_v(t0 + 3 < t_max ? t0 + 3 : t_max, (2 * P + 3) % 4);
     {
       PReg pb[PS];
-      if (!LAST) qk((2 * P + 2) % 4, s_a);
-      softmax_exp(s_b, pb);
+      qk_and_exp(std::integral_constant<bool, !LAST>{}, (2 * P + 2) % 4, s_a, s_b, pb);
       pv(((2 * P + 1) % 4) * C::V_TILE, pb);
       if (TRACK && !LAST) row_max_and_rescale(s_a, t0 + 2);
     }
