@@ -25,7 +25,7 @@ if ROOT not in sys.path:
 PEAK_TFLOPS = {"f16": 2500.0, "f8": 5000.0, "f32": 157.3}   # MI355X published dense MFMA peaks
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the same
 # counter reads for a plain 256 MiB copy: FETCH x2.0, WRITE x1.0); summaries are under profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"cfg2": (196971 + 67584) * 1024, "cfg4": (98535 + 65536) * 1024, "cfg5": (1575016 + 131072) * 1024}
+MEASURED_TRAFFIC_BYTES = {"cfg2": (196975 + 67584) * 1024, "cfg4": (98528 + 65536) * 1024, "cfg5": (1575016 + 131072) * 1024}
 
 WORKLOADS = {
     "cfg1": dict(kind="fmha", dtype="f16", B=1, H=8, S=512, D=64, scale=0.125),
