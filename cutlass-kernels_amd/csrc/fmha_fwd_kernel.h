@@ -396,6 +396,17 @@ fmha_fwd_kernel(const FmhaArgs a) {
     }
     l_run += rs;
   };
+  // the e4m3 V^T operand of K-step ps, d block db: four transpose reads (see the file comment)
+  auto read_v8 = [&](uint32_t vt, int ps, int db) __attribute__((always_inline)) -> int8v {
+    int8v va;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int2v x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(int2v, vt + v_rd[db] + (ps * 64 + u * 16) * C::V_PITCH));
+      va[2 * u] = x[0];
+      va[2 * u + 1] = x[1];
+    }
+    return va;
+  };
   // O^T += V^T . P^T for the V tile in LDS stage `stage`
   auto pv = [&](uint32_t vt /* byte offset of the V slot */, const PReg (&pb)[PS]) __attribute__((always_inline)) {
     if constexpr (MFMA_SUM) {
@@ -404,6 +415,19 @@ fmha_fwd_kernel(const FmhaArgs a) {
         if constexpr (PV8) l_acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(sum_a, pb[ps], l_acc, 0, 0, 0, 0, 0, 0);
         else l_acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(sum_a, pb[ps], l_acc, 0, 0, 0);
       }
+    }
+    if constexpr (PV8 && !C::VT && C::WPE == 2) {
+      // two waves per SIMD: the operand of the next multiply is requested before the current multiply is issued, the
+      // order pinned (left to itself the compiler reads, waits and multiplies one operand at a time: +0.8 %)
+      int8v ring[2];
+      ring[0] = read_v8(vt, 0, 0);
+#pragma unroll
+      for (int f = 0; f < PS * DB; ++f) {
+        if (f + 1 < PS * DB) ring[(f + 1) & 1] = read_v8(vt, (f + 1) / DB, (f + 1) % DB);
+        oacc[f % DB] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ring[f & 1], pb[f / DB], oacc[f % DB], 0, 0, 0, 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      return;
     }
 #pragma unroll
     for (int ps = 0; ps < PS; ++ps)
@@ -415,13 +439,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
           const int8v va = int8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb[ps], oacc[db], 0, 0, 0, 0, 0, 0);
         } else if constexpr (PV8) {
-          int8v va;
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const int2v x = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_AT(int2v, vt + v_rd[db] + (ps * 64 + u * 16) * C::V_PITCH));
-            va[2 * u] = x[0];
-            va[2 * u + 1] = x[1];
-          }
+          const int8v va = read_v8(vt, ps, db);
           oacc[db] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, pb[ps], oacc[db], 0, 0, 0, 0, 0, 0);
         } else {
           const uint32_t vp = vt + v_rd[db] + ps * 16 * C::V_PITCH;
