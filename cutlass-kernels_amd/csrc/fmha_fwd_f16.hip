@@ -29,6 +29,8 @@ using N128_128x64 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 1, 0, tru
 using N128_256x64 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 1, 0, true>;
 using N128_256x128 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 2, 0, true>;
 using N128_128x128 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 2, 0, true>;
+// ... and with the hand-scheduled main loop (key length a multiple of 256, at least 512)
+using A128_256x128 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 2, 0, true, true>;
 
 // builds that also write the score tap (debug): 128-row tile only
 using C64Tap = FmhaCfg<64, 64, 4, 2, false, false, false, true>;
@@ -36,7 +38,7 @@ using C128Tap = FmhaCfg<128, 64, 4, 2, false, false, false, true>;
 using C256Tap = FmhaCfg<256, 32, 4, 1, false, false, false, true>;
 
 using All64 = CfgList<C64_128x64, N64_128x64, C64_256x64, C64_128x128, C64_256x128>;
-using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128, N128_128x128, N128_256x128>;
+using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128, N128_128x128, A128_256x128, N128_256x128>;
 
 template <class F>
 bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
@@ -50,7 +52,7 @@ bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
   }
   switch (head_dim) {
     case 64: select_tile<All64, CfgList<N64_128x64, C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
-    case 128: select_tile<All128, CfgList<N128_256x128, N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
+    case 128: select_tile<All128, CfgList<A128_256x128, N128_256x128, N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
     default: return false;
   }
 }

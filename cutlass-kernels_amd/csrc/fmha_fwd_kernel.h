@@ -70,10 +70,11 @@ typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int2v __attribute__((ext_vector_type(2)));
 
 template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_, bool VT_ = false, bool TAP_S_ = false, int SUB_ = 1, int KPRE_ = 0,
-          bool M16_ = false>
+          bool M16_ = false, bool ASM_ = false>
 struct FmhaCfg {
   static constexpr int D = D_, BN = BN_, NWAVES = NWAVES_;
   static constexpr bool M16 = M16_;                             // the fp16 kernel on 16x16x32 MFMAs (fmha_fwd_kernel16.h)
+  static constexpr bool ASM = ASM_;                             // ... with the hand-scheduled main loop (gen_fmha_loop16.py)
   static constexpr int SUB = SUB_;                              // BN-key sub-tiles per barrier (1 or 2)
   static constexpr int KPRE = KPRE_;                            // K fragments of the next step read before the barrier
   static constexpr int NSLOT = KPRE ? 4 : 2 * SUB;              // LDS slots of one BN-key sub-tile of K
@@ -99,6 +100,7 @@ struct FmhaCfg {
   static_assert(D == 64 || D == 128 || D == 256, "head dim");
   static_assert(SUB == 1 || SUB == 2, "sub-tiles per barrier");
   static_assert(!KPRE || SUB == 1, "K fragment prefetch is a variant of the one-tile step");
+  static_assert(!ASM || (M16 && D == 128 && BN == 64 && NWAVES == 8 && SUB == 2 && WPE == 2), "the hand-scheduled loop exists for one shape");
   static_assert(BN % 32 == 0 && (!PV8 || BN == 64), "key tile: the e4m3 second GEMM has 64-deep K-steps");
   static_assert(!VT || PV8, "the pre-transposed layout is an e4m3-V layout");
   static_assert(K_IPW >= 1 && K_IPW * K_RPI * NWAVES == BN && V_IPW >= 1 && V_IPW * V_RPI * NWAVES == V_ROWS,
@@ -740,24 +742,30 @@ void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
 
 // ---- tile selection.  The reference fixes its tile at compile time (-DQBLKSIZE / -DKBLKSIZE,
 // src/fmha-pipeline/shared_storage.h:4-15, swept by compile_run_all_config.sh:3-6); here every shape is built and one is
-// picked per call.  CFK_FMHA_TILE=<query rows>x<keys>[/16|/32] (e.g. 256x128, or 256x64/16 for the build on 16x16x32
-// MFMAs), or small | large for the query rows alone, states a wish; a wish no instantiation can serve for the given
-// shape is ignored.
+// picked per call.  CFK_FMHA_TILE=<query rows>x<keys>[/16|/16h|/32] (e.g. 256x128, or 256x64/16 for the build on
+// 16x16x32 MFMAs, 256x128/16h for the one with the hand-scheduled main loop), or small | large for the query rows
+// alone, states a wish; a wish no instantiation can serve for the given shape is ignored.  CFK_FMHA_HANDLOOP=0 keeps
+// the automatic choice off the hand-scheduled builds (for A/B measurements).
 struct TileWish {
   int bm, bn;  // 0 = no wish
   int mfma;    // 16 or 32: the MFMA shape of the build (fp16 kernels come in both); 0 = no wish
+  int hand;    // +1: the build with the hand-scheduled loop, -1: a compiler-scheduled build, 0 = no wish
 };
 inline TileWish tile_wish() {
   static const TileWish w = [] {
-    TileWish t{0, 0, 0};
+    TileWish t{0, 0, 0, 0};
     const char *e = getenv("CFK_FMHA_TILE");
     if (!e) return t;
     if (e[0] == 's') t.bm = 128;
     else if (e[0] == 'l') t.bm = 256;
     else {
       int bm = 0, bn = 0, mfma = 0;
-      const int n = sscanf(e, "%dx%d/%d", &bm, &bn, &mfma);
-      if (n >= 2) t = TileWish{bm, bn, n == 3 && (mfma == 16 || mfma == 32) ? mfma : 0};
+      char suffix = 0;
+      const int n = sscanf(e, "%dx%d/%d%c", &bm, &bn, &mfma, &suffix);
+      if (n >= 2) {
+        const bool shape = n >= 3 && (mfma == 16 || mfma == 32);
+        t = TileWish{bm, bn, shape ? mfma : 0, !shape ? 0 : (n == 4 && suffix == 'h') ? 1 : -1};
+      }
     }
     return t;
   }();
@@ -768,10 +776,11 @@ template <class... Cs>
 struct CfgList {};
 
 // the shapes an instantiation can run: whole query tiles, whole key steps (four key tiles per loop turn with the K
-// fragment prefetch, two with the two-tile step)
+// fragment prefetch and in the hand-scheduled loop, which also needs eight tiles to fill and drain; two with the
+// two-tile step)
 template <class C>
 constexpr bool fits(int sq, int skv) {
-  return sq % C::BM == 0 && skv % (C::BN * (C::KPRE ? 4 : C::SUB)) == 0;
+  return sq % C::BM == 0 && skv % (C::BN * (C::KPRE || C::ASM ? 4 : C::SUB)) == 0 && (!C::ASM || skv >= 8 * C::BN);
 }
 
 // Calls f with the first instantiation of the list that fits the shape and the wish.  Without a wish for the query
@@ -786,6 +795,7 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, bool big, TileWish w, F &&f) {
     if (w.bm ? C::BM != w.bm : ((C::BM > 128 || C::M16) && !big)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
     if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;
+    if (w.hand && C::ASM != (w.hand > 0)) return;
     f(c);
     done = true;
   };
@@ -800,7 +810,8 @@ void select_tile(int sq, int skv, int bh, F &&f) {
   const bool big = sq % 256 == 0 && (long long)bh * (sq / 256) >= 512;
   const TileWish w = tile_wish();
   if ((w.bm || w.bn) && first_fit(All{}, sq, skv, big, w, f)) return;
-  if (first_fit(Auto{}, sq, skv, big, TileWish{0, 0, 0}, f)) return;
+  static const bool no_hand = [] { const char *e = getenv("CFK_FMHA_HANDLOOP"); return e && e[0] == '0'; }();
+  if (first_fit(Auto{}, sq, skv, big, TileWish{0, 0, 0, no_hand ? -1 : 0}, f)) return;
   f(Fallback{});
 }
 
