@@ -1,6 +1,6 @@
 // FMHA forward, fp16 operands: tile shapes and dispatch.  The kernels are in fmha_fwd_kernel.h (32x32 MFMAs) and
 // fmha_fwd_kernel16.h (16x16x32 MFMAs).
-#include "fmha_fwd_kernel16.h"
+#include "fmha_fwd_kernel16p.h"
 
 namespace cfk {
 namespace {

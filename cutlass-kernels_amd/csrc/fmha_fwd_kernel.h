@@ -93,7 +93,8 @@ struct FmhaCfg {
   static constexpr int O_PITCH = D * 2 + 16;                    // epilogue: a wave's 32 fp16 output rows, padded
   static constexpr int STAGE_BYTES = NSLOT * K_TILE + NSLOT_V * V_TILE;
   static constexpr int O_BYTES = NWAVES * 32 * O_PITCH;
-  static constexpr int LDS_BYTES = STAGE_BYTES > O_BYTES ? STAGE_BYTES : O_BYTES;
+  // (the hand-scheduled build keeps 32 KB of output staging behind its rings: fmha_fwd_kernel16p.h)
+  static constexpr int LDS_BYTES = ASM ? STAGE_BYTES + 32768 : STAGE_BYTES > O_BYTES ? STAGE_BYTES : O_BYTES;
   // one wave-wide 16 B/lane copy moves 1 KB = RPI rows; IPW copies per wave and tile
   static constexpr int K_RPI = 1024 / K_PITCH, K_IPW = BN / K_RPI / NWAVES;
   static constexpr int V_RPI = 1024 / V_PITCH, V_IPW = V_ROWS / V_RPI / NWAVES;
@@ -703,12 +704,26 @@ fmha_fwd_kernel(const FmhaArgs a) {
 // host threads), and callable ahead of any launch (cfk_init) so that a first call under stream capture finds it done.
 template <class C>
 __global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(C::WPE, C::WPE))) fmha_fwd_kernel16(const FmhaArgs a);
+template <class C>
+__global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(2, 2))) fmha_fwd_kernel16p(const FmhaArgs a);
 
 // the kernel an instantiation runs
 template <class C>
 constexpr auto fmha_kernel_of() {
-  if constexpr (C::M16) return &fmha_fwd_kernel16<C>;
+  if constexpr (C::ASM) return &fmha_fwd_kernel16p<C>;
+  else if constexpr (C::M16) return &fmha_fwd_kernel16<C>;
   else return &fmha_fwd_kernel<C>;
+}
+
+// Persistent workgroups (FmhaCfg::ASM): one per CU, a multiple of the 8 XCDs so that a workgroup's items stay on its XCD.
+inline int persistent_grid(int n_items) {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) n = 256;
+    return n / 8 * 8;
+  }();
+  const int g = n_items < cus ? n_items / 8 * 8 : cus;
+  return g < 8 ? n_items : g;
 }
 
 template <class C>
@@ -725,7 +740,8 @@ template <class C>
 hipError_t launch_fmha_cfg(const FmhaArgs &a, hipStream_t s) {
   const hipError_t e = prepare_fmha_cfg<C>();
   if (e != hipSuccess) return e;
-  const int grid = a.B * a.H * (a.Sq / C::BM);
+  const int items = a.B * a.H * (a.Sq / C::BM);
+  const int grid = C::ASM ? persistent_grid(items) : items;
   hipLaunchKernelGGL(fmha_kernel_of<C>(), dim3(grid), dim3(C::T), C::LDS_BYTES, s, a);
   return hipGetLastError();
 }

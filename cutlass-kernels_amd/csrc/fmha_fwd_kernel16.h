@@ -309,113 +309,7 @@ fmha_fwd_kernel16(const FmhaArgs a) {
 
   using std::integral_constant;
   f32x4 s_a[KB][QB], s_b[KB][QB];
-  if constexpr (C::ASM) {
-    // ---- The hand-scheduled loop (gen_fmha_loop16.py -> fmha_fwd_loop16_d128.inc): one asm statement that walks all key
-    // tiles with the softmax reference point fixed at the first tile's row max.  No rescale, no test per tile: a weight
-    // beyond the fp16 range (a score more than 16 binades above that max) turns l infinite, which is looked for once,
-    // after the loop; the workgroup then walks the keys again with the loop below, which follows the running max.
-    bool redo = want_taps;  // the taps want the true running max
-    if (!redo) {
-      const uint32_t tile_stride = (uint32_t)BN * k_ld;
-      load_k(0, 0);
-      load_v(0, 0);
-      load_k(1, 1);
-      load_k(2, 2);
-      load_v(1, 1);
-      wait_lds_dma();
-      __syncthreads();
-      qk(0, s_a);
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) {
-        const float mx = lane_max(s_a, qb);
-        float mfull = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mfull = fmaxf(mfull, __shfl_xor(mfull, 32, 64));
-        m_ref[qb] = mfull * c_log2;
-      }
-      __syncthreads();  // every wave is done with K slot 0 before the loop's first copies overwrite it
-      f32x16 sa0, sa1, q0v, q1v, o0, o1, o2, o3;
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        sa0[e] = s_a[e / 8][(e / 4) % 2][e % 4];
-        sa1[e] = s_a[2 + e / 8][(e / 4) % 2][e % 4];
-      }
-      {
-        half8 qh[2][4];
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) qh[qb][ks] = qreg[qb][ks];
-        __builtin_memcpy(&q0v, &qh[0][0], 64);
-        __builtin_memcpy(&q1v, &qh[1][0], 64);
-      }
-      uint64_t kptr = (uint64_t)(uintptr_t)Kp + 3ull * tile_stride, vptr = (uint64_t)(uintptr_t)Vp + 2ull * tile_stride;
-      uint32_t nloop = (uint32_t)(n_tiles / 2 - 4) / 2;
-      float l0, l1;
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-      asm volatile(
-#include "fmha_fwd_loop16_d128.inc"
-          : "={v[192:207]}"(o0), "={v[208:223]}"(o1), "={v[224:239]}"(o2), "={v[240:255]}"(o3), "={v42}"(l0), "={v43}"(l1),
-            "+{v[128:143]}"(sa0), "+{v[144:159]}"(sa1), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), [nloop] "+s"(nloop)
-          : "{v[96:111]}"(q0v), "{v[112:127]}"(q1v), "{v24}"(k_rd[0]), "{v25}"(k_rd[1]), "{v26}"(k_rd[2]), "{v27}"(k_rd[3]),
-            "{v28}"(v_rd[0]), "{v29}"(v_rd[1]), "{v30}"(v_rd[2]), "{v31}"(v_rd[3]), "{v32}"(v_rd[4]), "{v33}"(v_rd[5]),
-            "{v34}"(v_rd[6]), "{v35}"(v_rd[7]), "{v36}"(goff_k[0]), "{v37}"(goff_k[1]), "{v38}"(goff_v[0]), "{v39}"(goff_v[1]),
-            "{v40}"(m_ref[0]), "{v41}"(m_ref[1]), [c] "s"(c_log2), [ones] "s"(0x3c003c00u), [ldsw] "s"(lds_wave), [stride] "s"(tile_stride)
-          : "memory", "scc", "m0", "v44", "v45", "v46", "v47", "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58",
-            "v59", "v60", "v61", "v62", "v63", "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76",
-            "v77", "v78", "v79", "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94",
-            "v95", "v160", "v161", "v162", "v163", "v164", "v165", "v166", "v167", "v168", "v169", "v170", "v171", "v172", "v173",
-            "v174", "v175", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", "v187", "v188",
-            "v189", "v190", "v191");
-#pragma clang diagnostic pop
-      l_run[0] = l0;
-      l_run[1] = l1;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb)
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int e = 4 * (2 * db + qb) + t;
-            oacc[db][qb][t] = e < 16 ? o0[e] : e < 32 ? o1[e - 16] : e < 48 ? o2[e - 32] : o3[e - 48];
-          }
-      const bool bad = !(l0 < 3.0e38f) || !(l1 < 3.0e38f);
-      redo = __syncthreads_or(bad) != 0;  // (also: every wave is done with the LDS before the fallback refills it)
-    }
-    if (redo) {
-      // ---- The loop that follows the running max, tile by tile (online_softmax.h:123-165), not software-pipelined: taps,
-      // and scores that climbed out of the fp16 range of the weights.  K and V tiles alternate between two LDS slots.
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) oacc[db][qb] = zero4;
-#pragma unroll
-      for (int qb = 0; qb < QB; ++qb) m_ref[qb] = -INFINITY, m_lane[qb] = -INFINITY, l_run[qb] = 0.f;
-      load_k(0, 0);
-      load_v(0, 0);
-      for (int j = 0; j < n_tiles; ++j) {
-        const int st = j & 1;
-        wait_lds_dma();
-        __syncthreads();  // tile j has landed; every wave is done with the slots of tile j-1
-        if (j + 1 < n_tiles) {
-          load_k(j + 1, st ^ 1);
-          load_v(j + 1, st ^ 1);
-        }
-        qk(st, s_a);
-        rebase(s_a);
-        if (want_taps) {
-#pragma unroll
-          for (int qb = 0; qb < QB; ++qb) m_lane[qb] = __builtin_fmaxf(m_lane[qb], lane_max(s_a, qb));
-        }
-        half8 pb[QB][PS];
-        float rsum[QB];
-        exp_and_sum(s_a, pb, rsum);
-#pragma unroll
-        for (int qb = 0; qb < QB; ++qb) l_run[qb] += rsum[qb];
-        pv(st * C::V_TILE, pb);
-      }
-    }
-  } else if constexpr (C::SUB == 2) {
+  if constexpr (C::SUB == 2) {
     const int t_max = n_tiles - 1;
     load_k(0, 0);
     load_v(0, 0);

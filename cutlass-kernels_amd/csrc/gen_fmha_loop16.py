@@ -1,35 +1,46 @@
 #!/usr/bin/env python3
 """Generator of the hand-scheduled main loop of the fp16 FMHA forward kernel on 16x16x32 MFMAs
-(fmha_fwd_kernel16a.h), head dim 128, 256 query rows per workgroup (8 waves x 32 rows, two waves per SIMD).
+(fmha_fwd_kernel16.h, FmhaCfg::ASM), head dim 128, 256 query rows per workgroup (8 waves x 32 rows, two waves per SIMD).
 
     python3 gen_fmha_loop16.py            # rewrites fmha_fwd_loop16_d128.inc beside this file
+    python3 gen_fmha_loop16.py --check    # exit status 1 if that file is not what the generator produces
 
 Why a generator: the loop is one inline-asm statement of ~2800 instructions with every register assigned by hand.
 Left to the compiler, the step comes out as blocks (all MFMAs of a GEMM, then all of the softmax), the two waves of
 a SIMD run those blocks in lockstep and the matrix pipe idles during the softmax; at 256 registers any attempt to
 make it interleave spills.  Here each wave's instruction stream is uniform: every MFMA is followed by its share of
-the softmax's vector instructions (about 1.5 per MFMA) and of the LDS operand reads, operands are requested
-LOOKAHEAD fragments ahead through a ring of registers, and nothing spills.
+the softmax's vector instructions and of the LDS operand reads, operands are requested LOOKAHEAD fragments ahead
+through a ring of registers, and nothing spills.
 
-What the loop computes (same mathematics and data layout as fmha_fwd_kernel16.h; reference:
+What the vector pipe can take beside the MFMAs was measured with register-only loops (two waves per SIMD, cycles of
+the SIMD per v_mfma_f32_16x16x32_f16, 16.3 with nothing else): an MFMA holds the issue port for 8 cycles, an ordinary
+vector instruction for 4, v_exp_f32 for 8 -- up to two ordinary instructions per MFMA are free (16.5, 16.7), three
+are not (21.8), one exponential plus one multiply-add is not either (21.7); and a v_dot2c_f32_f16 between MFMAs
+waits for the matrix pipe to drain (32.5 with one per MFMA).  The softmax of a 64-key tile is 32 multiply-adds, 32
+exponentials and 16 packed converts per wave beside 64 MFMAs: 7 of the 8 free cycles per MFMA.  The row sum
+therefore does not go through the vector pipe at all (ROWSUM = "mfma"): four more MFMAs per tile multiply P by an
+all-ones operand, which also leaves every lane with the complete sum of its query.
+
+What the loop computes (same mathematics and data layout as the rest of fmha_fwd_kernel16.h; reference:
 src/fmha-pipeline/fmha_consumer.h:8-73, online_softmax.h:87-207, fmha_pipe_ws.h:245-296):
   for key tile t (64 keys):  S(t)^T = K(t) . Q^T ;  P(t) = fp16(exp2(c S(t) - m)) ;  l += rowsum P(t) ;
                              O^T += V(t)^T . P(t)^T
 with the reference point m fixed by the first tile's row max (no rescale inside the loop: the caller checks l for
 overflow afterwards and falls back to a loop that tracks the max).  S(0) is computed by the caller.
 
-Timeline.  One MFMA "slot" = one v_mfma_f32_16x16x32_f16 (16 cycles of the matrix pipe).  Tile t owns 64 slots:
-  slots 64t+[0,32)   S(t+1) = K(t+1).Q^T      (4 K-steps x 4 key blocks x 2 query blocks)
-  slots 64t+[32,64)  O += V(t).P(t)           (2 K-steps x 8 d blocks x 2 query blocks)
-The vector work of softmax(t+1) is spread over slots 64t+[48,105): it starts when P(t)'s first half has been consumed
-(its registers are reused) and ends before slot 64t+112 needs P(t+1)'s second half.
-A super-step = two tiles = 128 slots = one s_barrier.  K and V tiles live in rings of four 16 KB LDS slots (tile t
-in slot t % 4); super-step J (tiles 2J, 2J+1) issues the global->LDS copies of K tiles 2J+3, 2J+4 and V tiles 2J+2,
-2J+3 into the slots that the previous super-step read.  The barrier of a super-step sits HOLD MFMAs before its end:
-those MFMAs have their operands in registers already and cover the LDS latency of the next super-step's first K
+Timeline.  One MFMA "slot" = one v_mfma_f32_16x16x32_f16 (16 cycles of the matrix pipe).  Tile t owns T slots:
+  slots T t + [0,32)    S(t+1) = K(t+1).Q^T      (4 K-steps x 4 key blocks x 2 query blocks)
+  then per key half ps  O += V(t).P(t)           (8 d blocks x 2 query blocks), followed, with ROWSUM = "mfma", by
+                        l += 1.P(t)              (2 query blocks)
+The vector work of softmax(t+1) is spread evenly over one tile period starting at slot VALU_START of tile t's
+period: it starts when P(t)'s first half has been consumed (its registers are reused) and ends before P(t+1)'s second
+half is needed.  A super-step = two tiles = one s_barrier.  K and V tiles live in rings of four 16 KB LDS slots (tile
+t in slot t % 4); super-step J (tiles 2J, 2J+1) issues the global->LDS copies of K tiles 2J+3, 2J+4 and V tiles
+2J+2, 2J+3 into the slots that the previous super-step read.  The barrier of a super-step sits HOLD MFMAs before its
+end: those MFMAs have their operands in registers already and cover the LDS latency of the next super-step's first K
 fragments, which may only be read after the barrier.
 
-Registers (VGPRs, fixed):
+Registers (VGPRs, fixed; the generated file holds the whole asm statement with its constraints):
   v[192:255] O^T accumulators   o[db][qb]  at 192 + 4 (2 db + qb)
   v[128:159] S set A            s[kb][qb]  at base + 4 (2 kb + qb)     (even tiles)
   v[160:191] S set B                                                    (odd tiles)
@@ -38,11 +49,11 @@ Registers (VGPRs, fixed):
   v[48:79]   operand ring, 8 fragments of 4 registers (a K fragment = one ds_read_b128, a V fragment = two
              ds_read_b64_tr_b16); each fragment feeds two MFMAs (query blocks 0 and 1)
   v[24:27] K read addresses per K-step, v[28:35] V read addresses per d block, v[36:37] / v[38:39] lane offsets of
-  the K / V copies, v[40:41] m per query block, v[42:43] l, v[44:45] / v[46:47] the two partial row sums of the tile
+  the K / V copies; the softmax reference point m per query block and the row-sum registers depend on ROWSUM (below)
 SGPRs: s[40:41] / s[42:43] global address of the next K / V tile to copy; the rest are compiler-chosen operands.
 """
+import json
 import os
-import re
 import sys
 
 # ---- shape (head dim 128, 64-key tiles, 8 waves) ---------------------------------------------------------------
@@ -54,16 +65,38 @@ NSLOT = 4
 K_ST0, V_ST0 = 0, NSLOT * K_TILE        # LDS map: K slots, then V slots (the read addresses include these bases)
 IPW = 2                                  # copies per wave and tile (K and V alike)
 
+# ---- how the row sum l is taken ----------------------------------------------------------------------------------
+#   "mfma": l += 1 . P on the matrix pipe (sums P as rounded to fp16, the weights the second GEMM applies)
+#   "add":  v_add_f32 over the fp32 weights before the cast (online_softmax.h:173-206), two chains per query block
+#   "dot":  v_dot2c_f32_f16 over the rounded weights, summed per tile in the order of fmha_fwd_kernel16.h's loop
+ROWSUM = "add"
 # ---- registers ---------------------------------------------------------------------------------------------------
 O0, SA0, SB0, Q0, P0, RING0 = 192, 128, 160, 96, 80, 48
-KRD0, VRD0, GOK0, GOV0, M0R, L0, RS0, RS20 = 24, 28, 36, 38, 40, 42, 44, 46
+KRD0, VRD0, GOK0, GOV0 = 24, 28, 36, 38
 RING = 8
 LOOKAHEAD = 7      # fragments requested ahead of use
-HOLD = 8           # MFMAs of a super-step issued behind its barrier
-VALU_START = 48    # slot (within the previous tile's period) where softmax(t) starts
-VALU_RATE = 2.25   # issue slots (4 cycles each; v_exp_f32 counts two) per MFMA slot
+HOLD = 4           # MFMAs of a super-step issued behind its barrier
+VALU_START = None  # slot (within the previous tile's period) where softmax(t) starts; None: per ROWSUM
+VALU_RATE = None   # issue slots (4 cycles; v_exp_f32 counts two) per MFMA slot; None: even over one tile period
 # Ablation switches for timing experiments (the results are then wrong); never set in the committed include.
 ABLATE = set(os.environ.get("LOOP16_ABLATE", "").split(",")) - {""}
+
+
+def configure():
+    """derived constants; call again after changing ROWSUM or a parameter"""
+    g = globals()
+    if ROWSUM == "mfma":
+        g.update(M0R=18, ONES0=20, LACC0=40, QOFF0=16, LOW=16, L_OUT=(40, 44), T=68, L_TOTAL=True)
+        start = 46
+    elif ROWSUM == "add":
+        g.update(M0R=40, LA0=42, QOFF0=22, LOW=22, L_OUT=(42, 44), T=64, L_TOTAL=False)
+        start = 44
+    else:
+        g.update(M0R=40, L0=42, RS0=44, RS20=46, QOFF0=22, LOW=22, L_OUT=(42, 43), T=64, L_TOTAL=False)
+        start = 44
+    g["PV0"] = [32 + ps * (16 + (2 if ROWSUM == "mfma" else 0)) for ps in range(PS)]   # first slot of each key half's P.V
+    g["V_START"] = start if VALU_START is None else VALU_START
+    g["V_RATE"] = sum(c for _, c in softmax_ops(0)) / float(T) if VALU_RATE is None else VALU_RATE
 
 
 def o_reg(db, qb): return O0 + 4 * (2 * db + qb)
@@ -95,6 +128,11 @@ class Frag:
         return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (vr(d), vr(self.reg), vr(p_reg(qb, self.a)), vr(d))
 
 
+def sum_mfma(ps, qb):
+    d = LACC0 + 4 * qb
+    return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (vr(d), vr(ONES0), vr(p_reg(qb, ps)), vr(d))
+
+
 def softmax_ops(t):
     """vector instructions of softmax(t) in issue order: (text, issue slots)"""
     ops = []
@@ -104,20 +142,24 @@ def softmax_ops(t):
             p = p_reg(qb, kb // 2) + 2 * (kb % 2)
             for i in range(4): ops.append(("v_fma_f32 v%d, v%d, %%[c], -v%d" % (s + i, s + i, M0R + qb), 1))
             for i in range(4): ops.append(("v_exp_f32 v%d, v%d" % (s + i, s + i), 2))
+            if ROWSUM == "add":
+                for i in range(4): ops.append(("v_add_f32 v%d, v%d, v%d" % (LA0 + 2 * qb + i % 2, LA0 + 2 * qb + i % 2, s + i), 1))
             ops.append(("v_cvt_pk_f16_f32 v%d, v%d, v%d" % (p, s, s + 1), 1))
             ops.append(("v_cvt_pk_f16_f32 v%d, v%d, v%d" % (p + 1, s + 2, s + 3), 1))
-            if kb == 0:  # the tile's partial sums start from zero (same order of summation as fmha_fwd_kernel16.h)
-                ops.append(("v_dot2_f32_f16 v%d, %%[ones], v%d, 0" % (RS0 + qb, p), 1))
-                ops.append(("v_dot2_f32_f16 v%d, %%[ones], v%d, 0" % (RS20 + qb, p + 1), 1))
-            else:
-                ops.append(("v_dot2c_f32_f16 v%d, %%[ones], v%d" % (RS0 + qb, p), 1))
-                ops.append(("v_dot2c_f32_f16 v%d, %%[ones], v%d" % (RS20 + qb, p + 1), 1))
+            if ROWSUM == "dot":
+                if kb == 0:  # the tile's partial sums start from zero
+                    ops.append(("v_dot2_f32_f16 v%d, %%[ones], v%d, 0" % (RS0 + qb, p), 1))
+                    ops.append(("v_dot2_f32_f16 v%d, %%[ones], v%d, 0" % (RS20 + qb, p + 1), 1))
+                else:
+                    ops.append(("v_dot2c_f32_f16 v%d, %%[ones], v%d" % (RS0 + qb, p), 1))
+                    ops.append(("v_dot2c_f32_f16 v%d, %%[ones], v%d" % (RS20 + qb, p + 1), 1))
     return ops
 
 
 def tile_sum_ops():
-    """l += (rs + rs2) per query block; issued a few instructions after the tile's last v_dot2c"""
+    """ROWSUM = "dot": l += (rs + rs2) per query block; issued a few instructions after the tile's last v_dot2c"""
     ops = []
+    if ROWSUM != "dot": return ops
     for qb in range(QB): ops.append(("v_add_f32 v%d, v%d, v%d" % (RS0 + qb, RS0 + qb, RS20 + qb), 1))
     for qb in range(QB): ops.append(("v_add_f32 v%d, v%d, v%d" % (L0 + qb, L0 + qb, RS0 + qb), 1))
     return ops
@@ -139,34 +181,36 @@ def schedule(n_tiles):
     """straight-line program for n_tiles key tiles (a multiple of 4, at least 8), as a list of segments, one per
     super-step; a segment ends with its barrier (the last one has none)"""
     assert n_tiles % 4 == 0 and n_tiles >= 8
-    n_slots = 64 * n_tiles
+    n_slots = T * n_tiles
     n_steps = n_tiles // 2
-    # ---- MFMA slots and fragments
-    slot_frag = [None] * n_slots           # slot -> (frag, qb)
+    SS = 2 * T   # slots per super-step
+    # ---- MFMA slots: slot -> (fragment, qb) or ("L", ps, qb)
+    slot_item = [None] * n_slots
     frags = []
     for t in range(n_tiles):
-        base = 64 * t
+        base = T * t
         if t + 1 < n_tiles:
             for s in range(KS):
                 for kb in range(KB):
                     f = Frag('K', t + 1, s, kb, base + 2 * (s * KB + kb), len(frags)); frags.append(f)
-                    for qb in range(QB): slot_frag[f.slot0 + qb] = (f, qb)
+                    for qb in range(QB): slot_item[f.slot0 + qb] = (f, qb)
         for ps in range(PS):
             for db in range(DB):
-                f = Frag('V', t, ps, db, base + 32 + 2 * (ps * DB + db), len(frags)); frags.append(f)
-                for qb in range(QB): slot_frag[f.slot0 + qb] = (f, qb)
+                f = Frag('V', t, ps, db, base + PV0[ps] + 2 * db, len(frags)); frags.append(f)
+                for qb in range(QB): slot_item[f.slot0 + qb] = (f, qb)
+            if ROWSUM == "mfma":
+                for qb in range(QB): slot_item[base + PV0[ps] + 2 * DB + qb] = ("L", ps, qb)
     # ---- vector work: slot -> [text]; positions before slot 0 are issued ahead of it
     valu_at = {}
     for t in range(n_tiles):
-        start = 64 * (t - 1) + VALU_START
-        ops = softmax_ops(t)
+        start = T * (t - 1) + V_START
         cum = 0.0
-        for i, (txt, cost) in enumerate(ops):
-            valu_at.setdefault(max(int(start + cum / VALU_RATE), -1), []).append(txt)
+        for txt, cost in softmax_ops(t):
+            valu_at.setdefault(max(int(start + cum / V_RATE), -1), []).append(txt)
             cum += cost
         # the tile's sums join l a few instructions into the next tile's softmax (or right after, for the last tile)
         for txt, cost in tile_sum_ops():
-            valu_at.setdefault(max(int(start + cum / VALU_RATE) + 2, -1), []).append(txt)
+            valu_at.setdefault(max(int(start + cum / V_RATE) + 2, -1), []).append(txt)
     # ---- copies: super-step J, one copy instruction group every fourth slot from its second slot on
     copies_at = {}
     for J in range(n_steps):
@@ -174,10 +218,21 @@ def schedule(n_tiles):
         groups = []
         for kind, t in todo:
             if t < n_tiles: groups += copy_ops(kind, t % NSLOT)
-        for i, g in enumerate(groups): copies_at[128 * J + 1 + 4 * i] = g
+        for i, grp in enumerate(groups): copies_at[SS * J + 1 + 4 * i] = grp
+    # ---- the workgroup's next work item (persistent workgroups): in the last super-step, whose K slots 0-2 and V slots
+    # 0-1 are free, copy that item's first three K and two V tiles into them and, once the last S = K.Q^T has been
+    # issued, load its Q into the Q registers; both are waited for at the end of the statement
+    Z = SS * (n_steps - 1)
+    copies_at.setdefault(Z, [])
+    copies_at[Z] = ["s_mov_b64 s[40:41], %[kn]", "s_mov_b64 s[42:43], %[vn]"]
+    groups = []
+    for kind, slot in (('K', 0), ('K', 1), ('K', 2), ('V', 0), ('V', 1)): groups += copy_ops(kind, slot)
+    for i, grp in enumerate(groups): copies_at[Z + 1 + 4 * i] = grp
+    for i in range(QB * KS):
+        qb, ks = i // KS, i % KS
+        copies_at.setdefault(Z + 33 + 3 * i, []).append("global_load_dwordx4 %s, v%d, %%[qn] offset:%d" % (vr(q_reg(qb, ks)), QOFF0 + qb, 64 * ks))
     # ---- emission
     segs, cur = [], []
-    issued = []           # fragments whose reads have been issued, in order
     nread = 0             # LDS read instructions issued so far
     done_reads = 0        # ... known complete (by the last wait)
     read_end = {}         # frag idx -> nread after its last read
@@ -187,50 +242,63 @@ def schedule(n_tiles):
         # a K fragment of tile t >= 2 (first read in super-step (t-1)/2) needs the barrier of the super-step before
         if f.kind != 'K' or f.t < 2: return True
         J = (f.t - 1) // 2
-        return slot > 128 * J - HOLD   # `slot` is the slot after the MFMA just issued
+        return slot > SS * J - HOLD   # `slot` is the slot after the MFMA just issued
     def request(slot, limit):
         nonlocal next_frag, nread
         n = 0
         while next_frag < len(frags) and n < limit:
             f = frags[next_frag]
-            cur_frag = slot // 2
             # ring entry free: the fragment RING places earlier has been consumed (both MFMAs issued)
             if next_frag >= RING and frags[next_frag - RING].slot0 + 1 >= slot: break
-            if f.slot0 // 2 > cur_frag + LOOKAHEAD: break
+            if f.slot0 > slot + 2 * LOOKAHEAD: break
             if not barrier_passed_for(f, slot): break
             for r in f.reads():
                 if "reads" not in ABLATE: cur.append(r); nread += 1
             read_end[f.idx] = nread
             next_frag += 1; n += 1
     # ahead of slot 0: first operand requests, then the vector work that precedes the timeline
-    cur.append("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    cur.append("s_waitcnt lgkmcnt(0)")
     cur.append("s_nop 7"); cur.append("s_nop 7")   # MFMA results of the caller's S(0) are read by vector instructions
     for r in range(O0, O0 + 64): cur.append("v_mov_b32 v%d, 0" % r)
-    for qb in range(QB): cur.append("v_mov_b32 v%d, 0" % (L0 + qb))
+    if ROWSUM == "mfma":
+        for r in range(ONES0, ONES0 + 4): cur.append("v_mov_b32 v%d, 0x3c003c00" % r)
+        for r in range(LACC0, LACC0 + 8): cur.append("v_mov_b32 v%d, 0" % r)
+    elif ROWSUM == "add":
+        for r in range(LA0, LA0 + 4): cur.append("v_mov_b32 v%d, 0" % r)
+    else:
+        for qb in range(QB): cur.append("v_mov_b32 v%d, 0" % (L0 + qb))
+    if "reads" in ABLATE:
+        for r in range(RING0, RING0 + 4 * RING): cur.append("v_mov_b32 v%d, 0" % r)
     request(0, LOOKAHEAD)
     for txt in valu_at.get(-1, []): cur.append(txt)
     for slot in range(n_slots):
-        J = slot // 128
-        if slot % 128 == 128 - HOLD and J < n_steps - 1:
+        J = slot // SS
+        if slot % SS == SS - HOLD and J < n_steps - 1:
             cur.append("s_waitcnt lgkmcnt(0)" if "vmwait" in ABLATE else "s_waitcnt vmcnt(0) lgkmcnt(0)")
             if "barrier" not in ABLATE: cur.append("s_barrier")
             done_reads = nread
             segs.append(cur); cur = []
-        sf = slot_frag[slot]
-        if sf is not None and "mfma" not in ABLATE:
-            f, qb = sf
-            if qb == 0 and read_end[f.idx] > done_reads:
-                out = nread - read_end[f.idx]
-                assert out <= 15
-                if "reads" not in ABLATE: cur.append("s_waitcnt lgkmcnt(%d)" % out)
-                done_reads = read_end[f.idx]
-            cur.append(f.mfma(qb))
+        it = slot_item[slot]
+        if it is not None and "mfma" not in ABLATE:
+            if it[0] == "L":
+                cur.append(sum_mfma(it[1], it[2]))
+            else:
+                f, qb = it
+                if qb == 0 and read_end[f.idx] > done_reads:
+                    out = nread - read_end[f.idx]
+                    assert out <= 15
+                    if "reads" not in ABLATE: cur.append("s_waitcnt lgkmcnt(%d)" % out)
+                    done_reads = read_end[f.idx]
+                cur.append(f.mfma(qb))
         if "valu" not in ABLATE:
             for txt in valu_at.get(slot, []): cur.append(txt)
         request(slot + 1, 1)
         if "copies" not in ABLATE:
             for txt in copies_at.get(slot, []): cur.append(txt)
     assert next_frag == len(frags)
+    if ROWSUM == "add":
+        for qb in range(QB): cur.append("v_add_f32 v%d, v%d, v%d" % (LA0 + 2 * qb, LA0 + 2 * qb, LA0 + 2 * qb + 1))
+    cur.append("s_waitcnt vmcnt(0)")               # the next item's Q (registers) and first tiles (LDS) have arrived
     cur.append("s_nop 7"); cur.append("s_nop 7")   # the accumulators are read by the caller's vector instructions
     segs.append(cur)
     assert len(segs) == n_steps
@@ -256,11 +324,19 @@ def program(n_tiles):
 
 
 def render():
+    """the C++ text of the include: a flag the caller needs, then the complete asm statement.  It expects these names
+    in scope: f32x16 o0..o3 (out), sa0, sa1 (in, clobbered), q0v, q1v (in: this item's Q; out: the next item's); float
+    l0, l1 (out); uint64_t kptr, vptr (in: this item's K tile 3 / V tile 2; out: the same of the next item), kn, vn, qn
+    (the next item's K, V and this wave's Q rows); uint32_t nloop, k_rd[4], v_rd[8], goff_k[2], goff_v[2], qoff[2],
+    lds_wave, tile_stride; float m_ref[2], c_log2."""
     head, body, tail = folded()
-    lines = []
-    lines.append("// GENERATED by gen_fmha_loop16.py -- do not edit.  The hand-scheduled main loop of fmha_fwd_kernel16a (head dim")
-    lines.append("// 128, 256 x 128): %d + %d (loop) + %d instructions.  Operands: see the asm statement in fmha_fwd_kernel16a.h." % (len(head), len(body), len(tail)))
-    def emit(ins): lines.append('"%s\\n"' % ins)
+    L = []
+    L.append("// GENERATED by gen_fmha_loop16.py -- do not edit.  The hand-scheduled main loop of fmha_fwd_kernel16 (FmhaCfg::ASM: head")
+    L.append("// dim 128, 256 x 128): %d + %d (loop) + %d instructions, row sum by \"%s\"." % (len(head), len(body), len(tail), ROWSUM))
+    L.append("// l0 / l1 hold the complete row sum of the lane's query in every lane (true) or the lane's share of it (false)")
+    L.append("constexpr bool kLoop16SumIsComplete = %s;" % ("true" if L_TOTAL else "false"))
+    L.append("asm volatile(")
+    def emit(ins): L.append('    "%s\\n"' % ins)
     for i in head: emit(i)
     emit("s_cmp_eq_u32 %[nloop], 0")
     emit("s_cbranch_scc1 2f")
@@ -271,13 +347,28 @@ def render():
     emit("s_cbranch_scc1 1b")
     emit("2:")
     for i in tail: emit(i)
-    return "\n".join(lines) + "\n"
+    used = set(range(O0, O0 + 64)) | set(range(SA0, SA0 + 32)) | set(range(Q0, Q0 + 32)) | set(range(KRD0, GOV0 + 2)) | {M0R, M0R + 1, QOFF0, QOFF0 + 1} | set(L_OUT)
+    L.append('    : "={v[192:207]}"(o0), "={v[208:223]}"(o1), "={v[224:239]}"(o2), "={v[240:255]}"(o3), "={v%d}"(l0), "={v%d}"(l1),' % L_OUT)
+    L.append('      "+{v[128:143]}"(sa0), "+{v[144:159]}"(sa1), "+{v[96:111]}"(q0v), "+{v[112:127]}"(q1v), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), [nloop] "+s"(nloop)')
+    ins = ['"{v%d}"(qoff[%d])' % (QOFF0 + i, i) for i in range(QB)] + ['[kn] "s"(kn)', '[vn] "s"(vn)', '[qn] "s"(qn)']
+    ins += ['"{v%d}"(k_rd[%d])' % (KRD0 + i, i) for i in range(KS)] + ['"{v%d}"(v_rd[%d])' % (VRD0 + i, i) for i in range(DB)]
+    ins += ['"{v%d}"(goff_k[%d])' % (GOK0 + i, i) for i in range(IPW)] + ['"{v%d}"(goff_v[%d])' % (GOV0 + i, i) for i in range(IPW)]
+    ins += ['"{v%d}"(m_ref[%d])' % (M0R + i, i) for i in range(QB)]
+    ins += ['[c] "s"(c_log2)', '[ldsw] "s"(lds_wave)', '[stride] "s"(tile_stride)']
+    if ROWSUM == "dot": ins.append('[ones] "s"(0x3c003c00u)')
+    L.append("    : " + ", ".join(ins))
+    clob = ['"memory"', '"scc"', '"m0"'] + ['"v%d"' % r for r in range(LOW, 256) if r not in used]
+    L.append("    : " + ", ".join(clob) + ");")
+    return "\n".join(L) + "\n"
 
 
+configure()
 if __name__ == "__main__":
+    for k, v in json.loads(os.environ.get("LOOP16_SET", "{}")).items(): globals()[k] = v
+    configure()
     out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fmha_fwd_loop16_d128.inc")
     txt = render()
     if "--check" in sys.argv:
-        sys.exit(0 if open(out).read() == txt else 1)
+        sys.exit(0 if os.path.exists(out) and open(out).read() == txt else 1)
     open(out, "w").write(txt)
     print("wrote", out, len(txt.splitlines()), "lines")

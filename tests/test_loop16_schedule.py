@@ -49,17 +49,22 @@ class Checker:
         self.m0 = None
         self.m0_idx = -10
         self.kptr, self.vptr = 3, 2
+        self.next_item = {"s40": False, "s42": False}   # the pointer walks the next work item's tiles
+        self.vm_pending = False                          # a load with a register destination is in flight
         self.kparts, self.vparts = set(), set()
         self.kslot = {0: 0, 1: 1, 2: 2, 3: None}
         self.vslot = {0: 0, 1: 1, 2: None, 3: None}
         self.inflight = []    # copies issued since the last barrier: (kind, slot, tile)
         self.seg_reads = set()
         self.waited_all = False
-        self.n_mfma = 0
+        self.n_mfma = self.n_qk = 0
         for qb in range(g.QB):
             for s in range(g.KS):
                 for i in range(4): self.put(g.q_reg(qb, s) + i, ("Q", qb, s, i), 10 ** 9, "init")
             self.put(g.M0R + qb, ("m", qb), 10 ** 9, "init")
+            self.put(g.QOFF0 + qb, ("qoff", qb), 10 ** 9, "init")
+        self.e_need = 2 if g.ROWSUM == "add" else 1                 # uses of an exponential: the convert (+ the add)
+        self.p_need = g.DB + (0 if g.ROWSUM == "add" else 1)        # uses of a packed weight: 8 MFMAs (+ the row sum)
         for kb in range(g.KB):
             for qb in range(g.QB):
                 for i in range(4): self.put(g.s_reg(0, kb, qb) + i, ("S", 0, kb, qb, g.KS - 1, i), 1, "init")
@@ -106,9 +111,11 @@ class Checker:
                 continue
             if op == "s_waitcnt":
                 m = re.search(r"lgkmcnt\((\d+)\)", rest)
-                n = int(m.group(1))
-                assert n <= 15
-                self.complete = max(self.complete, self.nread - n)
+                n = int(m.group(1)) if m else None
+                if n is not None:
+                    assert n <= 15
+                    self.complete = max(self.complete, self.nread - n)
+                if "vmcnt(0)" in rest: self.vm_pending = False
                 self.waited_all = "vmcnt(0)" in rest and n == 0
             elif op == "s_barrier":
                 assert self.waited_all, "barrier without a full wait in front"
@@ -117,8 +124,8 @@ class Checker:
                     (self.kslot if kind == "K" else self.vslot)[slot] = t
                 self.inflight, self.seg_reads = [], set()
             elif op == "v_mov_b32":
-                assert a[1] == "0"
-                self.put(int(a[0][1:]), ("zero",), 10 ** 9, "valu")
+                assert a[1] in ("0", "0x3c003c00")
+                self.put(int(a[0][1:]), ("zero",) if a[1] == "0" else ("one",), 10 ** 9, "valu")
             elif op == "ds_read_b128":
                 lo, hi = R(a[0])
                 assert hi == lo + 3 and lo % 4 == 0
@@ -159,14 +166,14 @@ class Checker:
                 d, s_ = int(a[0][1:]), int(a[1][1:])
                 tag = self.get(s_, "valu")
                 assert d == s_ and tag[0] == "X", ins
-                self.put(d, ("E",) + tag[1:], 1, "trans")
+                self.put(d, ("E",) + tag[1:], self.e_need, "trans")
             elif op == "v_cvt_pk_f16_f32":
                 d = int(a[0][1:])
                 ta, tb = self.get(int(a[1][1:]), "valu"), self.get(int(a[2][1:]), "valu")
                 assert ta[0] == "E" and tb[0] == "E" and ta[1:4] == tb[1:4] and ta[4] % 2 == 0 and tb[4] == ta[4] + 1, ins
                 t, kb, qb, j = ta[1], ta[2], ta[3], ta[4] // 2
                 assert d == g.p_reg(qb, kb // 2) + 2 * (kb % 2) + j, ins
-                self.put(d, ("Ph", t, qb, kb, j), g.DB + 1, "valu")
+                self.put(d, ("Ph", t, qb, kb, j), self.p_need, "valu")
             elif op in ("v_dot2_f32_f16", "v_dot2c_f32_f16"):
                 d = int(a[0][1:])
                 assert a[1] == "%[ones]"
@@ -187,7 +194,19 @@ class Checker:
                 d, x, y = (int(s[1:]) for s in a)
                 assert d == x
                 tx, ty = self.get(x, "valu"), self.get(y, "valu")
-                if tx[0] == "rs":
+                if g.ROWSUM == "add":
+                    if ty[0] == "E":      # l chain j of query block qb takes elements j, j+2 of every block, in order
+                        t, kb, qb, i = ty[1:]
+                        assert d == g.LA0 + 2 * qb + i % 2, ins
+                        cnt = 0 if tx == ("zero",) else tx[3]
+                        assert tx == ("zero",) or tx[:3] == ("la", qb, i % 2)
+                        assert cnt == (t * g.KB + kb) * 2 + i // 2, "weights summed out of order (%s)" % ins
+                        self.put(d, ("la", qb, i % 2, cnt + 1), 10 ** 9, "valu")
+                    else:                 # the two chains of a query block meet after the last tile
+                        full = self.n * g.KB * 2
+                        assert tx[0] == "la" and ty[0] == "la" and tx[1] == ty[1] and (tx[2], ty[2]) == (0, 1) and tx[3] == full and ty[3] == full, ins
+                        self.put(d, ("l", tx[1], self.n), 10 ** 9, "valu")
+                elif tx[0] == "rs":
                     full = tuple(range(g.KB))
                     assert ty[0] == "rs" and tx[1:3] == ty[1:3] and (tx[3], ty[3]) == (0, 1) and tx[4] == full and ty[4] == full, ins
                     self.put(d, ("rsum", tx[1], tx[2]), 1, "valu")
@@ -209,7 +228,11 @@ class Checker:
                 assert rel % (g.NWAVES * 1024) == 0 and part < g.IPW and gt == ("gok" if kind == "K" else "gov", part), ins
                 assert a[1] == ("s[40:41]" if kind == "K" else "s[42:43]")
                 t = self.kptr if kind == "K" else self.vptr
-                assert t < self.n and slot == t % g.NSLOT, "copy of tile %d into slot %d (%s)" % (t, slot, ins)
+                if self.next_item["s40" if kind == "K" else "s42"]:
+                    assert t < (3 if kind == "K" else 2) and slot == t, "next item: copy of tile %d into slot %d (%s)" % (t, slot, ins)
+                    t = ("next", t)   # no MFMA of this program may read it
+                else:
+                    assert t < self.n and slot == t % g.NSLOT, "copy of tile %d into slot %d (%s)" % (t, slot, ins)
                 assert (kind, slot) not in self.seg_reads, "%s slot %d read and then copied into in one barrier interval" % (kind, slot)
                 parts = self.kparts if kind == "K" else self.vparts
                 assert part not in parts
@@ -224,6 +247,22 @@ class Checker:
                 parts.clear()
                 if sp == "s40": self.kptr += 1
                 else: self.vptr += 1
+            elif op == "s_mov_b64":
+                sp = {"s[40:41]": "s40", "s[42:43]": "s42"}[a[0]]
+                assert a[1] == ("%[kn]" if sp == "s40" else "%[vn]")
+                assert (self.kptr if sp == "s40" else self.vptr) == self.n, "pointer handed to the next item before this item's copies are out"
+                assert not (self.kparts if sp == "s40" else self.vparts)
+                self.next_item[sp] = True
+                if sp == "s40": self.kptr = 0
+                else: self.vptr = 0
+            elif op == "global_load_dwordx4":
+                lo, hi = R(a[0])
+                addr, off = a[2].split(" offset:")
+                qt = self.get(int(a[1][1:]), "vmem")
+                assert addr == "%[qn]" and qt[0] == "qoff" and hi == lo + 3 and lo == g.q_reg(qt[1], int(off) // 64) and int(off) % 64 == 0, ins
+                assert self.n_qk == 32 * (self.n - 1), "Q overwritten before the last S = K.Q^T was issued"
+                for i in range(4): self.put(lo + i, ("Qnext", qt[1], int(off) // 64, i), 10 ** 9, "vmem")
+                self.vm_pending = True
             elif op == "s_addc_u32":
                 assert a[0] == a[1] and a[2] == "0" and a[0] in ("s41", "s43")
             else:
@@ -235,12 +274,24 @@ class Checker:
         self.n_mfma += 1
         ta = [self.get(a + i, "mfma") for i in range(4)]
         tb = [self.get(b + i, "mfma") for i in range(4)]
-        if ta[0][0] == "Kf":
+        if ta[0] == ("one",):
+            assert ta == [("one",)] * 4 and a == g.ONES0, self.cur
+            _, t, qb, kb0, _ = tb[0]
+            ps = kb0 // 2
+            assert tb == [("Ph", t, qb, 2 * ps + j // 2, j % 2) for j in range(4)] and b == g.p_reg(qb, ps), self.cur
+            assert d == g.LACC0 + 4 * qb and c == d, self.cur
+            tc = [self.get(d + i, "mfma_c") for i in range(4)]
+            n_prev = 0 if tc[0] == ("zero",) else tc[0][2]
+            assert all(x == ("zero",) for x in tc) or tc == [("lacc", qb, n_prev, i) for i in range(4)], self.cur
+            assert n_prev == 2 * t + ps, "row sum takes tile %d half %d as its %d-th term" % (t, ps, n_prev)
+            for i in range(4): self.put(d + i, ("lacc", qb, n_prev + 1, i), 1, "mfma")
+        elif ta[0][0] == "Kf":
             _, t, s, kb, _ = ta[0]
             assert ta == [("Kf", t, s, kb, i) for i in range(4)], self.cur
             qb = tb[0][1]
             assert tb == [("Q", qb, s, i) for i in range(4)] and b == g.q_reg(qb, s), self.cur
             assert d == g.s_reg(t, kb, qb), self.cur
+            self.n_qk += 1
             if s == 0:
                 assert c is None, self.cur
             else:
@@ -265,17 +316,29 @@ class Checker:
         for db in range(g.DB):
             for qb in range(g.QB):
                 for i in range(4): assert self.v[g.o_reg(db, qb) + i].tag == ("O", db, qb, 2 * n, i)
-        for qb in range(g.QB): assert self.v[g.L0 + qb].tag == ("l", qb, n)
-        assert self.n_mfma == 32 * (n - 1) + 32 * n
-        assert self.kptr == n and self.vptr == n and not self.kparts and not self.vparts
+        for qb in range(g.QB):
+            if g.ROWSUM == "mfma": assert self.v[g.L_OUT[qb]].tag == ("lacc", qb, 2 * n, 0)
+            else: assert self.v[g.L_OUT[qb]].tag == ("l", qb, n)
+        assert self.n_mfma == 32 * (n - 1) + (g.T - 32) * n
+        # the next work item: its first three K and two V tiles are on their way into slots 0-2 / 0-1, its Q is in the Q
+        # registers, and everything has been waited for
+        assert self.next_item == {"s40": True, "s42": True} and self.kptr == 3 and self.vptr == 2 and not self.kparts and not self.vparts
+        assert sorted((k, s, t) for k, s, t in self.inflight) == [("K", i, ("next", i)) for i in range(3)] + [("V", i, ("next", i)) for i in range(2)]
+        assert not self.vm_pending
+        for qb in range(g.QB):
+            for ks in range(g.KS):
+                for i in range(4): assert self.v[g.q_reg(qb, ks) + i].tag == ("Qnext", qb, ks, i)
         # the accumulators are read by the caller right after the statement
         last_mfma = max(v.widx for v in self.v.values() if v.wkind == "mfma")
         assert self.idx - last_mfma > 8
 
 
+@pytest.mark.parametrize("rowsum", ["mfma", "add", "dot"])
 @pytest.mark.parametrize("n_tiles", [8, 12, 16, 32, 64])
-def test_loop_is_correct_symbolically(n_tiles):
+def test_loop_is_correct_symbolically(n_tiles, rowsum):
     g = _gen()
+    g.ROWSUM = rowsum
+    g.configure()
     c = Checker(g, n_tiles)
     c.run(g.program(n_tiles))
     c.finish()

@@ -2,8 +2,9 @@
 the tile wish CFK_FMHA_TILE, read once per process by the library -- and prints one JSON line per case with the
 tile the library planned and the errors against the CPU oracle.
 
-usage: tile_case.py mode:B,S,H,D[,Skv] ...      mode = f16 | f8 | hyb, with the suffix `climb` for keys whose scores
-climb along the key axis (tests/_util.py: climbing_keys)
+usage: tile_case.py mode:B,S,H,D[,Skv] ...      mode = f16 | f16nt | f8 | hyb, with the suffix `climb` for keys whose
+scores climb along the key axis (tests/_util.py: climbing_keys); f16nt = fp16 without the row taps (the hand-scheduled
+build serves calls with taps through its max-tracking loop: only a call without them runs the scheduled loop)
 """
 import json
 import sys
@@ -25,13 +26,16 @@ def run_case(spec):
         mode, k, v = mode[:-5], climbing_keys(k), v / 4
     f = pkg.fmha
     mfma = 32
+    no_taps = mode == "f16nt"
+    if no_taps: mode = "f16"
     if mode == "f16":
         q16, k16, v16 = (x.astype(np.float16) for x in (q, k, v))
         plan = f.fmha_forward_plan(f.CFK_FP16, B, H, S, Skv, D)
         mfma = f.fmha_forward_mfma(f.CFK_FP16, B, H, S, Skv, D)
         rm = torch.full((B, H, S), -1.0, dtype=torch.float32, device="cuda:0")
         rs = torch.full((B, H, S), -1.0, dtype=torch.float32, device="cuda:0")
-        o = pkg.fmha_forward(to_dev(q16), to_dev(k16), to_dev(v16), row_max=rm, row_sum=rs)
+        if no_taps: o = pkg.fmha_forward(to_dev(q16), to_dev(k16), to_dev(v16))
+        else: o = pkg.fmha_forward(to_dev(q16), to_dev(k16), to_dev(v16), row_max=rm, row_sum=rs)
         qf, kf, vf = (x.astype(np.float32) for x in (q16, k16, v16))
     else:
         (qc, qs), (kc, ks) = oracle.quantize_e4m3_per_tensor(q), oracle.quantize_e4m3_per_tensor(k)
@@ -57,7 +61,7 @@ def run_case(spec):
     sel = ~np.isnan(ref)
     _, pct = oracle.verify_tensor(got[sel], ref[sel])
     taps = None
-    if mode == "f16":
+    if mode == "f16" and not no_taps:
         # the row-max / row-sum taps of the first and last (batch, head): log2-domain max, sum not reciprocal
         st = oracle.attention_f32(qf, kf, vf, bh_pairs=pairs, want_stats=True)
         m_ref, inv_ref = st["row_max"], st["inv_sum"]
