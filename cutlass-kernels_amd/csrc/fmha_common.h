@@ -21,7 +21,11 @@ struct FmhaArgs {
   float s_scale;     // softmax_scale * q_descale * k_descale (scales the score tap)
   int32_t v_layout;  // 0 = [B,S,H,D], 1 = [B,D,H,S]
   float tau;         // the softmax reference point moves when a tile's max exceeds it by more than this (log2 domain)
+  int32_t track_only;  // no optimistic first pass over the keys (cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, 1))
 };
+
+// cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, ...): also steers the choice of instantiation (fmha_fwd_kernel.h: select_tile)
+bool predictable_latency();
 
 struct FmhaPlan {
   int32_t block_m, block_n, lds_bytes, threads, grid;

@@ -649,7 +649,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
 
   };
   // (fp16 P gains nothing from the first pass -- its row max hides behind the second GEMM's MFMAs -- and skips it.)
-  bool redo = !PV8 || C::TAP_S || a.row_max != nullptr || a.row_sum != nullptr || !(kTau > 0.f);
+  bool redo = !PV8 || C::TAP_S || a.row_max != nullptr || a.row_sum != nullptr || !(kTau > 0.f) || a.track_only != 0;
   if (!redo) {
     pass(integral_constant<bool, false>{});
     const float l_chk = MFMA_SUM ? l_acc[0] : l_run;
@@ -827,7 +827,8 @@ void select_tile(int sq, int skv, int bh, F &&f) {
   const TileWish w = tile_wish();
   if ((w.bm || w.bn) && first_fit(All{}, sq, skv, big, w, f)) return;
   static const bool no_hand = [] { const char *e = getenv("CFK_FMHA_HANDLOOP"); return e && e[0] == '0'; }();
-  if (first_fit(Auto{}, sq, skv, big, TileWish{0, 0, 0, no_hand ? -1 : 0}, f)) return;
+  // (the hand-scheduled build is a two-pass kernel: not for callers that asked for a data-independent run time)
+  if (first_fit(Auto{}, sq, skv, big, TileWish{0, 0, 0, no_hand || predictable_latency() ? -1 : 0}, f)) return;
   f(Fallback{});
 }
 

@@ -142,7 +142,7 @@ def softmax_ops(t):
             p = p_reg(qb, kb // 2) + 2 * (kb % 2)
             for i in range(4): ops.append(("v_fma_f32 v%d, v%d, %%[c], -v%d" % (s + i, s + i, M0R + qb), 1))
             for i in range(4): ops.append(("v_exp_f32 v%d, v%d" % (s + i, s + i), 2))
-            if ROWSUM == "add":
+            if ROWSUM == "add" and "rowsum" not in ABLATE:
                 for i in range(4): ops.append(("v_add_f32 v%d, v%d, v%d" % (LA0 + 2 * qb + i % 2, LA0 + 2 * qb + i % 2, s + i), 1))
             ops.append(("v_cvt_pk_f16_f32 v%d, v%d, v%d" % (p, s, s + 1), 1))
             ops.append(("v_cvt_pk_f16_f32 v%d, v%d, v%d" % (p + 1, s + 2, s + 3), 1))
@@ -172,7 +172,7 @@ def copy_ops(kind, slot):
     ops = []
     for i in range(IPW):
         ops.append(["s_add_u32 m0, %%[ldsw], %d" % (base + i * NWAVES * 1024), "s_nop 0",
-                    "global_load_lds_dwordx4 v%d, s[%d:%d]" % (go + i, sp, sp + 1)])
+                    "global_load_lds_dwordx4 v%d, s[%d:%d]%s" % (go + i, sp, sp + 1, os.environ.get("LOOP16_COPYMOD", ""))])
     ops[-1] += ["s_add_u32 s%d, s%d, %%[stride]" % (sp, sp), "s_addc_u32 s%d, s%d, 0" % (sp + 1, sp + 1)]
     return ops
 

@@ -347,9 +347,12 @@ int main(int argc, char **argv) {
   if (opt.streams > 1)
     for (auto &s : streams) HIP_CHECK(hipStreamCreate(&s));
   const int Lb = B / opt.streams;
-  void *dout_tap = nullptr;  // O of the score-tap launch (a debug build of the kernel): only gemm-check-1 uses that launch
-  if (check_scores) HIP_CHECK(hipMalloc(&dout_tap, n * 2));
-  // taps: 0 = none, 1 = row max / row sum (the kernel that was timed), 2 = scores as well (debug build, O discarded)
+  // O of the launches with taps: those launches only serve max-check / sum-check (taps = 1) and gemm-check-1 (taps = 2, a
+  // debug build of the kernel); a kernel may take another path through its code when taps are asked for, so the output
+  // that is checked and dumped is the timed launches' own
+  void *dout_tap = nullptr;
+  if (check_scores || opt.verify_all) HIP_CHECK(hipMalloc(&dout_tap, n * 2));
+  // taps: 0 = none (the launches that are timed), 1 = row max / row sum, 2 = scores (debug build)
   auto launch_all = [&](int iters, int taps) -> int {
     for (int it = 0; it < iters; ++it)
       for (int i = 0; i < opt.streams; ++i) {
@@ -358,7 +361,7 @@ int main(int argc, char **argv) {
         p.q = (const char *)dq + off * esz;
         p.k = (const char *)dk + off * esz;
         p.v = (const char *)dv + off * vesz;
-        p.o = (taps == 2 ? (char *)dout_tap : (char *)dout) + off * 2;
+        p.o = (taps != 0 ? (char *)dout_tap : (char *)dout) + off * 2;
         p.q_descale = descale[0];
         p.k_descale = descale[1];
         p.v_descale = descale[2];
@@ -392,12 +395,14 @@ int main(int argc, char **argv) {
   const double t = ms_total / 1e3 / opt.iterations;
   printf("CUTE_FMHA:     [%6.1f]Gflop/s  (%6.4f)ms\n", fmha_flops / t, t * 1000);  // line format of :595-597
 
-  // one more launch of the SAME kernel with the row taps on: O, row max and row sum checked below come from it
-  if (launch_all(1, 1) != 0) return 2;
-  if (check_scores && launch_all(1, 2) != 0) return 2;  // scores: separate launch of the debug build
+  // the output that is checked (gemm-check-2) and dumped: what the last timed launch wrote
   HIP_CHECK(hipDeviceSynchronize());
   std::vector<_Float16> ho(n);
   HIP_CHECK(hipMemcpy(ho.data(), dout, n * 2, hipMemcpyDeviceToHost));
+  // separate launches for the taps, into an O buffer of their own
+  if (opt.verify_all && launch_all(1, 1) != 0) return 2;
+  if (check_scores && launch_all(1, 2) != 0) return 2;
+  HIP_CHECK(hipDeviceSynchronize());
 
   if (!opt.dump_dir.empty()) {
     bool ok = write_file(opt.dump_dir + "/q.bin", qb.data(), qb.size()) && write_file(opt.dump_dir + "/k.bin", kb.data(), kb.size()) &&

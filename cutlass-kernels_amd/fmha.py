@@ -22,6 +22,7 @@ CFK_V_BSHD = 0
 CFK_V_BDHS = 1
 CFK_GEMM_TN = 0
 CFK_GEMM_NN = 1
+CFK_OPT_PREDICTABLE_LATENCY = 1
 
 
 class CfkError(RuntimeError):
@@ -88,6 +89,8 @@ def lib():
         l.cfk_gemm.argtypes = [ctypes.POINTER(GemmParams), ctypes.c_void_p]
         l.cfk_init.restype = ctypes.c_int
         l.cfk_init.argtypes = []
+        l.cfk_set_option.restype = ctypes.c_int
+        l.cfk_set_option.argtypes = [ctypes.c_int32, ctypes.c_int32]
         l.cfk_last_error.restype = ctypes.c_char_p
         l.cfk_version.restype = ctypes.c_char_p
         _lib = l
@@ -97,6 +100,11 @@ def lib():
 def init() -> None:
     """``cfk_init``: one-time set-up of every kernel on the current device (optional; launches do it on demand)."""
     _check(lib().cfk_init())
+
+
+def set_option(option: int, value: int) -> None:
+    """``cfk_set_option``: process-wide options, e.g. ``CFK_OPT_PREDICTABLE_LATENCY``."""
+    _check(lib().cfk_set_option(option, value))
 
 
 def last_error() -> str:

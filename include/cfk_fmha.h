@@ -35,7 +35,10 @@ typedef enum cfk_status {
 /* Operand precision; values mirror the driver flag --prec-type (src/fmha-pipeline/fmha_forward.cu:694,733). */
 typedef enum cfk_dtype { CFK_FP16 = 1, CFK_FP8_E4M3 = 2, CFK_FP32 = 3 /* GEMM only */ } cfk_dtype;
 
-/* Layout of V in memory. */
+/* Layout of V in memory.  Not accepted: the reference's third convention, -DFP8NOSHFL (fmha_forward.cu:534-558), which
+ * additionally permutes V's sequence index inside every block of 16 on the host so that its kernel needs no register
+ * shuffles.  The kernels here need neither the shuffles nor the permutation (the key order of P is applied where V is
+ * read from the LDS): a caller that keeps that host permutation must drop it, or O comes out wrong. */
 typedef enum cfk_v_layout {
   CFK_V_BSHD = 0, /* [B, S_kv, H, D], D contiguous -- the reference's default (fmha_forward.cu:189-190)       */
   CFK_V_BDHS = 1  /* [B, D, H, S_kv], S contiguous -- the reference's offline pre-transposed fp8 V (GEMM2FP8,
@@ -55,7 +58,7 @@ typedef struct cfk_fmha_fwd_params {
                         without -DGEMM2FP8 (fmha_forward.cu:446-450)                                            */
   int32_t batch;     /* BATCH                                                                                 */
   int32_t heads;     /* NUMHEADS                                                                              */
-  int32_t seqlen_q;  /* SEQLEN: multiple of 128                                                               */
+  int32_t seqlen_q;  /* SEQLEN: multiple of 128 (the query rows of a workgroup: 128 or 256)                   */
   int32_t seqlen_kv; /* KEYLEN: multiple of 64 (32 for fp16 V at head_dim 256); cfk_fmha_forward_plan reports the
                         key tile actually chosen                                                              */
   int32_t head_dim;  /* HEADDIM: 64, 128 or 256 (fmha_forward.cu:746-761)                                     */
@@ -97,7 +100,8 @@ int cfk_fmha_forward_plan(const cfk_fmha_fwd_params *params, int32_t *block_m, i
 /* The MFMA shape of the kernel build the library would pick for `params`: 32 (32x32x16 / 32x32x64 MFMAs) or 16
  * (16x16x32; fp16 operands, big problems at head dims 64 and 128: the more power-efficient shape on this board).  No
  * counterpart in the reference, whose MMA atom is fixed at compile time (src/fmha-pipeline/ss_helper.h:3-94).  The
- * environment variable CFK_FMHA_TILE=<query rows>x<keys>[/16|/32] overrides the automatic choice of tile and shape.
+ * environment variable CFK_FMHA_TILE=<query rows>x<keys>[/16|/16h|/32] overrides the automatic choice of tile and shape
+ * (16h: the 16x16x32 build with the hand-scheduled main loop and persistent workgroups, fp16 head dim 128).
  * Does not touch the GPU. */
 int cfk_fmha_forward_mfma(const cfk_fmha_fwd_params *params, int32_t *mfma_rows);
 
@@ -133,6 +137,19 @@ typedef struct cfk_gemm_params {
   void *d;
 } cfk_gemm_params;
 int cfk_gemm(const cfk_gemm_params *p, void *stream);
+
+/* Process-wide options (read by every later call; set them before launching from several threads).  No counterpart in the
+ * reference, whose choices of this kind are compile-time macros (src/fmha-pipeline/README.md:11-28). */
+typedef enum cfk_option {
+  /* 1: no optimistic first pass.  Two kernels first walk the keys with a softmax reference point fixed by the first key
+   * tile (no row max per tile) and, only if some weight left the range of P's type, walk them again tracking the running
+   * max as the reference does on every tile (online_softmax.h:123-165): e4m3 P from 2048 keys on, and fp16 at head dim
+   * 128 on big problems.  On scores that climb along the key axis that costs up to twice the time.  With this option
+   * every call takes the max-tracking path from the start: the same results to rounding, a run time that does not
+   * depend on the data (a few per cent slower on ordinary data).  0 (default): two passes where they pay. */
+  CFK_OPT_PREDICTABLE_LATENCY = 1
+} cfk_option;
+int cfk_set_option(int32_t option, int32_t value);
 
 /* Optional: performs the one-time per-process set-up of every kernel (raising their dynamic-LDS limits) on the
  * current device.  Launch calls do the same on first use of a kernel, thread-safely; calling this first keeps that

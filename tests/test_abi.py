@@ -129,3 +129,17 @@ def test_python_binding_refuses_cpu_tensors():
     x = torch.zeros((1, 128, 1, 64), dtype=torch.float16)
     with pytest.raises(ValueError):
         pkg.fmha_forward(x, x, x)
+
+
+def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
+    # big fp16 problems at head dim 128 run the two-pass build with the hand-scheduled loop (160 KB of LDS); with the option
+    # set the choice falls on the one-pass build (128 KB); unknown options are refused
+    f = pkg.fmha
+    assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:3] == (256, 128, 163840)
+    f.set_option(f.CFK_OPT_PREDICTABLE_LATENCY, 1)
+    try:
+        assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:3] == (256, 128, 131072)
+    finally:
+        f.set_option(f.CFK_OPT_PREDICTABLE_LATENCY, 0)
+    with pytest.raises(pkg.CfkError):
+        f.set_option(99, 1)

@@ -69,7 +69,7 @@ def _load_dump(d):
                                              (2, 128, ["--v-layout=bdhs"]), (2, 64, ["--v-layout=bdhs", "--fp8-scales=amax"])])
 def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
     # fp8 needs the reference's own sequence length for its percentage criterion; fp16 passes at any length
-    seq = 2048 if prec == 2 else 512
+    seq = 4096 if prec == 2 else 512   # (e4m3 P: the two-pass path starts at 4096 keys)
     out = _run(f"--prec-type={prec}", "--batch-size=2", f"--dim-size={2 * head}", f"--head-size={head}",
                f"--seq-length={seq}", "--iterations=3", "--reference-check=true", "--verify-all=true",
                f"--dump-dir={tmp_path}", *extra).stdout
@@ -96,7 +96,9 @@ def test_sweep_script_verify_all_on_a_reduced_problem():
     # run_all_config.sh (the counterpart of compile_run_all_config.sh) in its verify-all mode: every precision mode x
     # head size x tile shape that exists, each with gemm-check-1 / max-check / sum-check / gemm-check-2
     script = os.path.join(ROOT, "cutlass-kernels_amd", "driver", "run_all_config.sh")
-    env = dict(os.environ, BATCH="1", SEQ="2048", DIM="512")
+    # (the reference's own sequence length, 4096: its error-percentage gate is calibrated there, and the e4m3 kernel walks
+    # the keys in two passes from that length on -- the path its FLOP runs time)
+    env = dict(os.environ, BATCH="1", SEQ="4096", DIM="512")
     r = subprocess.run(["bash", script, "verify-all"], env=env, capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout[-4000:] + r.stderr[-2000:]
     blocks = r.stdout.split("CONFIG ")[1:]

@@ -84,8 +84,8 @@ def test_shortest_and_odd_key_tile_counts(B, S, H, D, Skv):
                                          (2, 2048, 32, 128, 2048)])
 def test_scores_that_climb_along_the_keys_move_the_reference_point(mode, B, S, H, D, Skv):
     # the deferred rescale's slow path, many times per row (e4m3 P has two binades of head-room above the row max of
-    # the moment, so here almost every tile takes it); with 2048 keys the e4m3 kernel starts in its pass without a row
-    # max per tile, finds non-finite rows and walks the keys again.  The last shape is large enough for the automatic
+    # the moment, so here almost every tile takes it); from 4096 keys on the e4m3 kernel starts in its pass without a row
+    # max per tile, finds non-finite rows and walks the keys again (the tests of the second pass below).  The last shape is large enough for the automatic
     # choice of the 256-row tile (two sub-tiles per barrier for e4m3 P).
     import torch
     from _util import TOL_FP16
@@ -343,3 +343,99 @@ def test_config4_subset_check():
           f"vs unquantised fp32 attention {max_abs(got[s1], full[s1]):.3e}")
     assert err <= TOL_FP8 and ok
     assert not np.any(np.isnan(got))
+
+
+# ---- the two-pass e4m3 kernel (from 4096 keys on): first pass without a row max per tile, second pass only where a
+# weight left the range of e4m3.  Every instantiation that can take the second pass is driven through it here.
+def _climb_case(B, S, H, D, Skv, v_layout=None, ramp=4.0, spike=8.0):
+    import torch
+    f = pkg.fmha
+    q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=Skv)
+    k, v = climbing_keys(k, ramp=ramp, spike=spike), v / 4
+    (qc, qs, qf), (kc, ks, kf), (vc, vs, vf) = _quant(q), _quant(k), _quant(v)
+    if v_layout == "bdhs":
+        vdev = to_dev(np.ascontiguousarray(vc.transpose(0, 3, 2, 1)))  # [B,S,H,D] -> [B,D,H,S]
+        o = pkg.fmha_forward(to_dev(qc), to_dev(kc), vdev, q_descale=qs, k_descale=ks, v_descale=vs, v_layout=f.CFK_V_BDHS)
+    else:
+        o = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(vc), q_descale=qs, k_descale=ks, v_descale=vs)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    pairs = sorted({(0, 0), (B - 1, H - 1)})
+    ref = oracle.attention_f32(qf, kf, vf, bh_pairs=pairs)["O"]
+    sel = ~np.isnan(ref)
+    err = max_abs(got[sel], ref[sel])
+    print(f"e4m3 climbing B={B} S={S}/{Skv} H={H} D={D} v_layout={v_layout}: max-abs {err:.3e}")
+    assert not np.isnan(got).any()
+    assert err <= TOL_FP8, err
+
+
+@pytest.mark.parametrize("B,S,H,D,Skv", [(1, 256, 2, 64, 4096), (1, 128, 3, 64, 4352), (1, 128, 2, 256, 4096), (1, 256, 1, 256, 4224)])
+def test_second_pass_at_head_dims_64_and_256(B, S, H, D, Skv):
+    # head dim 64 runs three waves per SIMD; head dim 256 has no row sum on the MFMA pipe: a non-finite O is all its
+    # detection has
+    _climb_case(B, S, H, D, Skv)
+
+
+@pytest.mark.parametrize("B,S,H,D,Skv", [(1, 256, 2, 64, 4096), (1, 256, 2, 128, 4096), (1, 128, 1, 256, 4096), (1, 256, 2, 128, 4608)])
+def test_second_pass_with_pretransposed_v(B, S, H, D, Skv):
+    _climb_case(B, S, H, D, Skv, v_layout="bdhs")
+
+
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("where", ["one_row_mid", "one_row_last_tile"])
+def test_second_pass_for_a_single_row(D, where):
+    # N(0,1) operands, except that ONE query row is a large multiple of ONE key -- in the middle of the key sequence, or
+    # in its last tile: that row's score there exceeds the first tile's max by far more than e4m3 P has room for, every
+    # other row of the workgroup (and every other workgroup) is ordinary.  The workgroup that owns the row takes the
+    # second pass; the result must be right for the row and for its neighbours.
+    import torch
+    B, S, H, Skv = 1, 256, 2, 4096
+    q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=Skv)
+    row, key = 77, (1000 if where == "one_row_mid" else Skv - 3)
+    q[0, row, 1] = 6.0 * k[0, key, 1]
+    (qc, qs, qf), (kc, ks, kf), (vc, vs, vf) = _quant(q), _quant(k), _quant(v)
+    o = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(vc), q_descale=qs, k_descale=ks, v_descale=vs)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    ref = oracle.attention_f32(qf, kf, vf)["O"]
+    err = max_abs(got, ref)
+    # the row itself: its softmax is one key
+    assert max_abs(got[0, row, 1], vf[0, key, 1]) <= TOL_FP8
+    print(f"e4m3 single climbing row D={D} {where}: max-abs {err:.3e}")
+    assert not np.isnan(got).any() and err <= TOL_FP8, err
+
+
+def test_both_sides_of_the_key_length_where_the_passes_change():
+    # below 2048 keys: one pass whose reference point follows the running max (tau = 0); from 2048 on it moves only when it
+    # must (deferred rescale); from 4096 on: two passes.  The same operands, cut on both sides of each boundary.
+    B, S, H, D = 1, 256, 2, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=4096)
+    for skv in (1984, 2048, 4032, 4096):
+        got, (qf, kf, vf) = _run(q, k[:, :skv], v[:, :skv])
+        ref = oracle.attention_f32(qf, kf, vf)["O"]
+        err, (ok, pct) = max_abs(got, ref), oracle.verify_tensor(got, ref, ERRPCT_FP8)
+        print(f"e4m3 S_kv={skv}: max-abs {err:.3e}, error% {pct:.2e}")
+        assert err <= TOL_FP8 and pct <= 2 * ERRPCT_FP8 + EMU_PCT_FLOOR, (skv, err, pct)
+
+
+def test_predictable_latency_option_takes_the_tracked_pass():
+    # cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, 1): straight to the pass that tracks the row max -- the pass a call
+    # with taps takes, so the two outputs are bit-identical; the default (two passes) agrees to rounding
+    import torch
+    f = pkg.fmha
+    B, S, H, D = 1, 256, 2, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=4096)
+    (qc, qs, qf), (kc, ks, kf), (vc, vs, vf) = _quant(q), _quant(k), _quant(v)
+    args = (to_dev(qc), to_dev(kc), to_dev(vc))
+    kw = dict(q_descale=qs, k_descale=ks, v_descale=vs)
+    o_default = pkg.fmha_forward(*args, **kw).float().cpu().numpy()
+    rm = torch.zeros((B, H, S), dtype=torch.float32, device="cuda:0")
+    o_taps = pkg.fmha_forward(*args, row_max=rm, **kw).float().cpu().numpy()
+    f.set_option(f.CFK_OPT_PREDICTABLE_LATENCY, 1)
+    try:
+        o_opt = pkg.fmha_forward(*args, **kw).float().cpu().numpy()
+    finally:
+        f.set_option(f.CFK_OPT_PREDICTABLE_LATENCY, 0)
+    assert np.array_equal(o_opt, o_taps)
+    ref = oracle.attention_f32(qf, kf, vf)["O"]
+    assert max_abs(o_default, ref) <= TOL_FP8 and max_abs(o_opt, ref) <= TOL_FP8
