@@ -23,9 +23,35 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"f16": 2500.0, "f8": 5000.0, "f32": 157.3}   # MI355X published dense MFMA peaks
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by what the same
-# counter reads for a plain 256 MiB copy: FETCH x2.0, WRITE x1.0); summaries are under profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"cfg2": (196975 + 67584) * 1024, "cfg4": (98528 + 65536) * 1024, "cfg5": (1575016 + 131072) * 1024}
+# HBM bytes per launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, two runs) and scaled by what
+# the same counters read for a plain device copy of known size in the same session.  Every figure names the profile it
+# was read from and the kernel it was read for: tests/test_bench_contract.py parses the figures out of those files and
+# checks that the kernel is the one the library picks for the workload, so a stale figure fails in the CPU suite.
+COPY_CALIBRATION = dict(profile="profiles/fmha_fwd_f16_B8_H16_S2048_D128.md", kernel="__amd_rocclr_copyBuffer",
+                        known_kib=262144, fetch_kib=131090, write_kib=262144)
+TRAFFIC_SOURCE = {
+    "cfg2": dict(profile="profiles/fmha_fwd_f16_B8_H16_S2048_D128.md", kernel="fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>",
+                 fetch_kib=110045, write_kib=69632),
+    "cfg3": dict(profile="profiles/fmha_fwd_f16_B2_H8_S8192_D256.md", kernel="fmha_fwd_kernel<256,32,4,1,0,0,0,0,1,4,0,0>",
+                 fetch_kib=164068, write_kib=65536),
+    "cfg4": dict(profile="profiles/fmha_fwd_fp8_B4_H16_S4096_D128.md", kernel="fmha_fwd_kernel<128,64,8,2,1,1,0,0,2,0,0,0>",
+                 fetch_kib=49260, write_kib=65536),
+    "cfg5": dict(profile="profiles/gemm_M8192_N8192_K8192.md", kernel="gemm_kernel16<0,4>", fetch_kib=787716, write_kib=131072),
+}
+
+
+def measured_traffic(workload):
+    """(HBM bytes per launch, where the figure comes from) or (None, None) for a workload that has no counter run."""
+    t = TRAFFIC_SOURCE.get(workload)
+    if t is None:
+        return None, None
+    c = COPY_CALIBRATION
+    kib = t["fetch_kib"] * c["known_kib"] / c["fetch_kib"] + t["write_kib"] * c["known_kib"] / c["write_kib"]
+    return int(round(kib * 1024)), {"profile": t["profile"], "kernel": t["kernel"], "FETCH_SIZE_KiB": t["fetch_kib"],
+                                    "WRITE_SIZE_KiB": t["write_kib"],
+                                    "fetch_scale": round(c["known_kib"] / c["fetch_kib"], 4),
+                                    "write_scale": round(c["known_kib"] / c["write_kib"], 4)}
+
 
 WORKLOADS = {
     "cfg1": dict(kind="fmha", dtype="f16", B=1, H=8, S=512, D=64, scale=0.125),
@@ -185,6 +211,7 @@ def main():
             except pkg.CfkError as e:
                 secondary.append({"workload": NAMES[name], "error": str(e)})
     w = WORKLOADS[args.workload]
+    traffic, traffic_source = measured_traffic(args.workload)
     out = {
         "metric": "fmha_fwd_tflops",
         "value": main_res["tflops"],
@@ -205,7 +232,7 @@ def main():
                                "untimed 0.4 s burst of launches that lets the clock governor settle; not in the reference"},
         "roofline": {"bound": "mfma", "achieved": main_res["tflops"], "peak": main_res["peak_tflops"],
                      "unit": "TFLOP/s", "frac": main_res["frac_of_peak"],
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload)},
+                     "traffic": traffic, "traffic_source": traffic_source},
         "secondary": secondary,
     }
     if not args.no_cpu_baseline and w["kind"] == "fmha":

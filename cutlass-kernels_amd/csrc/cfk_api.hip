@@ -117,6 +117,15 @@ int cfk_fmha_forward_mfma(const cfk_fmha_fwd_params *params, int32_t *mfma_rows)
   return CFK_OK;
 }
 
+int cfk_fmha_forward_kernel(const cfk_fmha_fwd_params *params, char *name, int32_t capacity) {
+  cfk::FmhaPlan plan{};
+  int rc = check_fmha(params, &plan, false);
+  if (rc != CFK_OK) return rc;
+  if (!name || capacity <= (int32_t)strlen(plan.kernel)) return fail(CFK_ERR_INVALID_ARG, "name buffer of %d bytes is too small", capacity);
+  memcpy(name, plan.kernel, strlen(plan.kernel) + 1);
+  return CFK_OK;
+}
+
 int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
   cfk::FmhaPlan plan{};
   int rc = check_fmha(p, &plan, true);

@@ -30,6 +30,7 @@ bool predictable_latency();
 struct FmhaPlan {
   int32_t block_m, block_n, lds_bytes, threads, grid;
   int32_t mfma;  // 32: 32x32 MFMA build, 16: 16x16x32 build
+  char kernel[80];  // the instantiation, as profilers print it without namespaces: fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>
 };
 
 // Each launcher validates nothing: the C-ABI layer has already checked shapes against the plan.

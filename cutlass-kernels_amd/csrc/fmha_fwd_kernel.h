@@ -93,7 +93,8 @@ struct FmhaCfg {
   static constexpr int O_PITCH = D * 2 + 16;                    // epilogue: a wave's 32 fp16 output rows, padded
   static constexpr int STAGE_BYTES = NSLOT * K_TILE + NSLOT_V * V_TILE;
   static constexpr int O_BYTES = NWAVES * 32 * O_PITCH;
-  // (the hand-scheduled build keeps 32 KB of output staging behind its rings: fmha_fwd_kernel16p.h)
+  // (the hand-scheduled build: 128 KB of K/V rings plus 32 KB; its 64 KB of output staging lie over the rings' upper
+  // slots and those 32 KB: fmha_fwd_kernel16p.h)
   static constexpr int LDS_BYTES = ASM ? STAGE_BYTES + 32768 : STAGE_BYTES > O_BYTES ? STAGE_BYTES : O_BYTES;
   // one wave-wide 16 B/lane copy moves 1 KB = RPI rows; IPW copies per wave and tile
   static constexpr int K_RPI = 1024 / K_PITCH, K_IPW = BN / K_RPI / NWAVES;
@@ -754,6 +755,9 @@ void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
   p->lds_bytes = C::LDS_BYTES;
   p->threads = C::T;
   p->grid = bh * (sq / C::BM);
+  snprintf(p->kernel, sizeof p->kernel, "%s<%d,%d,%d,%d,%d,%d,%d,%d,%d,%d,%d,%d>",
+           C::ASM ? "fmha_fwd_kernel16p" : C::M16 ? "fmha_fwd_kernel16" : "fmha_fwd_kernel", C::D, C::BN, C::NWAVES, C::WPE,
+           (int)C::QK8, (int)C::PV8, (int)C::VT, (int)C::TAP_S, C::SUB, C::KPRE, (int)C::M16, (int)C::ASM);
 }
 
 // ---- tile selection.  The reference fixes its tile at compile time (-DQBLKSIZE / -DKBLKSIZE,

@@ -83,6 +83,8 @@ def lib():
         l.cfk_fmha_forward_plan.argtypes = [ctypes.POINTER(FmhaFwdParams)] + [ctypes.POINTER(ctypes.c_int32)] * 4
         l.cfk_fmha_forward_mfma.restype = ctypes.c_int
         l.cfk_fmha_forward_mfma.argtypes = [ctypes.POINTER(FmhaFwdParams), ctypes.POINTER(ctypes.c_int32)]
+        l.cfk_fmha_forward_kernel.restype = ctypes.c_int
+        l.cfk_fmha_forward_kernel.argtypes = [ctypes.POINTER(FmhaFwdParams), ctypes.c_char_p, ctypes.c_int32]
         l.cfk_gemm_f16.restype = ctypes.c_int
         l.cfk_gemm_f16.argtypes = [ctypes.c_int32] * 3 + [ctypes.c_void_p] * 3 + [ctypes.c_int32, ctypes.c_void_p]
         l.cfk_gemm.restype = ctypes.c_int
@@ -151,6 +153,15 @@ def fmha_forward_mfma(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, v_layo
     out = ctypes.c_int32()
     _check(lib().cfk_fmha_forward_mfma(ctypes.byref(p), ctypes.byref(out)))
     return out.value
+
+
+def fmha_forward_kernel(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, v_layout=CFK_V_BSHD, v_dtype=None):
+    """``cfk_fmha_forward_kernel``: the name of the instantiation the library launches for this call, as a kernel trace
+    prints it (``fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>``).  No GPU needed."""
+    p = make_params(dtype, batch, heads, seqlen_q, seqlen_kv, head_dim, v_layout=v_layout, v_dtype=v_dtype)
+    buf = ctypes.create_string_buffer(80)
+    _check(lib().cfk_fmha_forward_kernel(ctypes.byref(p), buf, len(buf)))
+    return buf.value.decode()
 
 
 def _stream_ptr(stream):

@@ -105,6 +105,15 @@ int cfk_fmha_forward_plan(const cfk_fmha_fwd_params *params, int32_t *block_m, i
  * Does not touch the GPU. */
 int cfk_fmha_forward_mfma(const cfk_fmha_fwd_params *params, int32_t *mfma_rows);
 
+/* The name of the kernel instantiation the library would launch for `params`, as a profiler's kernel trace prints it
+ * without its namespaces and with the booleans as 0/1, e.g. "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>" (template
+ * arguments: head dim, keys per tile, waves, waves per SIMD, e4m3 QK, e4m3 PV, V pre-transposed, score tap, tiles per
+ * barrier, K fragment prefetch, 16x16x32 MFMAs, hand-scheduled loop): ties a measurement to the code that was measured.
+ * `name` receives a NUL-terminated string of fewer than 80 bytes; CFK_ERR_INVALID_ARG if `capacity` is too small.  No
+ * counterpart in the reference (one kernel per executable: src/fmha-pipeline/fmha_forward.cu:321-331).  Does not touch
+ * the GPU. */
+int cfk_fmha_forward_kernel(const cfk_fmha_fwd_params *params, char *name, int32_t capacity);
+
 /* GEMM layouts for cfk_gemm_f16. */
 typedef enum cfk_gemm_layout {
   CFK_GEMM_TN = 0, /* A: M x K (K contiguous), B: N x K (K contiguous) -- the reference's form
