@@ -106,4 +106,25 @@ __device__ __forceinline__ void lds_dma16(const void *base, uint32_t lane_off, u
 #pragma clang diagnostic pop
 __device__ __forceinline__ void wait_lds_dma() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// The lane number, computed on the spot (two v_mbcnt) from an operand the compiler cannot see through: neither kept in a
+// register across the main loop nor hoisted out of the item loop.
+__device__ __forceinline__ unsigned fresh_zero() {
+  unsigned z = 0;
+  asm volatile("" : "+v"(z));
+  return z;
+}
+__device__ __forceinline__ int fresh_lane() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, fresh_zero())); }
+
+// Exchange among the four lanes c, c+16, c+32, c+48 that share a query, without a lane number in a register and
+// without the LDS: v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its
+// second, v_permlane32_swap the same for 32-lane halves; with x in both operands the two results, combined, are the
+// pairwise max / sum.  (Written as asm: this compiler's builtin hands back the first result twice.  The s_nop covers
+// the wait states the instruction wants behind a vector write of its operands.)
+__device__ __forceinline__ void swap_rows16(float &a, float &b) {
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap_rows32(float &a, float &b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+}
+
 }  // namespace cfk

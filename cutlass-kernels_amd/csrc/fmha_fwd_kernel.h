@@ -94,15 +94,17 @@ struct FmhaCfg {
   static constexpr int STAGE_BYTES = NSLOT * K_TILE + NSLOT_V * V_TILE;
   static constexpr int O_BYTES = NWAVES * 32 * O_PITCH;
   // (the hand-scheduled build: 128 KB of K/V rings plus 32 KB; its 64 KB of output staging lie over the rings' upper
-  // slots and those 32 KB: fmha_fwd_kernel16p.h)
-  static constexpr int LDS_BYTES = ASM ? STAGE_BYTES + 32768 : STAGE_BYTES > O_BYTES ? STAGE_BYTES : O_BYTES;
+  // slots and those 32 KB: fmha_fwd_kernel16p.h;
+  // ... the e4m3 one 64 KB of its own behind its 64 KB of rings, and a dword for the vote: fmha_fwd_kernel8p.h)
+  static constexpr int LDS_BYTES = ASM ? (QK8 ? STAGE_BYTES + 65536 + 1024 : STAGE_BYTES + 32768) : STAGE_BYTES > O_BYTES ? STAGE_BYTES : O_BYTES;
   // one wave-wide 16 B/lane copy moves 1 KB = RPI rows; IPW copies per wave and tile
   static constexpr int K_RPI = 1024 / K_PITCH, K_IPW = BN / K_RPI / NWAVES;
   static constexpr int V_RPI = 1024 / V_PITCH, V_IPW = V_ROWS / V_RPI / NWAVES;
   static_assert(D == 64 || D == 128 || D == 256, "head dim");
   static_assert(SUB == 1 || SUB == 2, "sub-tiles per barrier");
   static_assert(!KPRE || SUB == 1, "K fragment prefetch is a variant of the one-tile step");
-  static_assert(!ASM || (M16 && D == 128 && BN == 64 && NWAVES == 8 && SUB == 2 && WPE == 2), "the hand-scheduled loop exists for one shape");
+  static_assert(!ASM || ((M16 != (QK8 && PV8 && !VT)) && QK8 == PV8 && D == 128 && BN == 64 && NWAVES == 8 && SUB == 2 && WPE == 2),
+                "the hand-scheduled loops exist for one shape: fp16 on 16x16x32 MFMAs, e4m3 with V in [B,S,H,D]");
   static_assert(BN % 32 == 0 && (!PV8 || BN == 64), "key tile: the e4m3 second GEMM has 64-deep K-steps");
   static_assert(!VT || PV8, "the pre-transposed layout is an e4m3-V layout");
   static_assert(K_IPW >= 1 && K_IPW * K_RPI * NWAVES == BN && V_IPW >= 1 && V_IPW * V_RPI * NWAVES == V_ROWS,
@@ -707,11 +709,14 @@ template <class C>
 __global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(C::WPE, C::WPE))) fmha_fwd_kernel16(const FmhaArgs a);
 template <class C>
 __global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(2, 2))) fmha_fwd_kernel16p(const FmhaArgs a);
+template <class C>
+__global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(2, 2))) fmha_fwd_kernel8p(const FmhaArgs a);
 
 // the kernel an instantiation runs
 template <class C>
 constexpr auto fmha_kernel_of() {
-  if constexpr (C::ASM) return &fmha_fwd_kernel16p<C>;
+  if constexpr (C::ASM && C::QK8) return &fmha_fwd_kernel8p<C>;
+  else if constexpr (C::ASM) return &fmha_fwd_kernel16p<C>;
   else if constexpr (C::M16) return &fmha_fwd_kernel16<C>;
   else return &fmha_fwd_kernel<C>;
 }
@@ -756,7 +761,7 @@ void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
   p->threads = C::T;
   p->grid = bh * (sq / C::BM);
   snprintf(p->kernel, sizeof p->kernel, "%s<%d,%d,%d,%d,%d,%d,%d,%d,%d,%d,%d,%d>",
-           C::ASM ? "fmha_fwd_kernel16p" : C::M16 ? "fmha_fwd_kernel16" : "fmha_fwd_kernel", C::D, C::BN, C::NWAVES, C::WPE,
+           C::ASM ? (C::QK8 ? "fmha_fwd_kernel8p" : "fmha_fwd_kernel16p") : C::M16 ? "fmha_fwd_kernel16" : "fmha_fwd_kernel", C::D, C::BN, C::NWAVES, C::WPE,
            (int)C::QK8, (int)C::PV8, (int)C::VT, (int)C::TAP_S, C::SUB, C::KPRE, (int)C::M16, (int)C::ASM);
 }
 
@@ -800,7 +805,8 @@ struct CfgList {};
 // two-tile step)
 template <class C>
 constexpr bool fits(int sq, int skv) {
-  return sq % C::BM == 0 && skv % (C::BN * (C::KPRE || C::ASM ? 4 : C::SUB)) == 0 && (!C::ASM || skv >= 8 * C::BN);
+  return sq % C::BM == 0 && skv % (C::BN * (C::KPRE || C::ASM ? 4 : C::SUB)) == 0 &&
+         (!C::ASM || skv >= (C::QK8 ? 64 : 8) * C::BN);
 }
 
 // Calls f with the first instantiation of the list that fits the shape and the wish.  Without a wish for the query

@@ -136,9 +136,14 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     # set the choice falls on the one-pass build (128 KB); unknown options are refused
     f = pkg.fmha
     assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:3] == (256, 128, 163840)
+    # ... and so do big e4m3 problems from 4096 keys (below, e4m3 weights always follow the running max: one pass)
+    assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128) == "fmha_fwd_kernel8p<128,64,8,2,1,1,0,0,2,0,0,1>"
+    assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 4, 16, 4096, 2048, 128) == "fmha_fwd_kernel<128,64,8,2,1,1,0,0,2,0,0,0>"
+    assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128, v_layout=f.CFK_V_BDHS) == "fmha_fwd_kernel<128,64,4,2,1,1,1,0,1,0,0,0>"
     f.set_option(f.CFK_OPT_PREDICTABLE_LATENCY, 1)
     try:
         assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:3] == (256, 128, 131072)
+        assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128) == "fmha_fwd_kernel<128,64,8,2,1,1,0,0,2,0,0,0>"
     finally:
         f.set_option(f.CFK_OPT_PREDICTABLE_LATENCY, 0)
     with pytest.raises(pkg.CfkError):

@@ -33,6 +33,10 @@ CASES = {
     # (half of the workgroups take a second item), 5x16x1024 = 320 with climbing keys (fall-back, then a next item)
     "256x128/16h": ["f16nt:1,512,2,128", "f16nt:1,256,3,128,768", "f16nt:2,2048,16,128", "f16nt:3,2048,16,128", "f16nt:1,512,2,128,1024",
                     "f16ntclimb:1,512,2,128,768", "f16ntclimb:5,1024,16,128", "f16:1,512,2,128", "f16:3,2048,16,128", "f16climb:1,512,2,128,768"],
+    # the e4m3 build with the hand-scheduled loop and persistent workgroups (key length a multiple of 256, from 4096): the
+    # scheduled loop, 4352 keys (an odd number of loop turns), 2x10 heads x 4096 rows = 320 items (a quarter of the
+    # workgroups take a second one), climbing keys (the vote, the max-tracking loop, then a next item: 5x13x1024 rows = 260)
+    "256x128/32h": ["f8:1,256,2,128,4096", "f8:1,512,1,128,4352", "f8:2,4096,10,128", "f8climb:1,256,2,128,4096", "f8climb:5,1024,13,128,4096"],
 }
 
 
