@@ -127,4 +127,19 @@ __device__ __forceinline__ void swap_rows32(float &a, float &b) {
   asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
 }
 
+__device__ __forceinline__ float quad_max(float x) {
+  float a = x, b = x;
+  swap_rows16(a, b);
+  a = b = fmaxf(a, b);
+  swap_rows32(a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float quad_sum(float x) {
+  float a = x, b = x;
+  swap_rows16(a, b);
+  a = b = a + b;
+  swap_rows32(a, b);
+  return a + b;
+}
+
 }  // namespace cfk

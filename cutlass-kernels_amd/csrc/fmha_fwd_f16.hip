@@ -1,6 +1,7 @@
 // FMHA forward, fp16 operands: tile shapes and dispatch.  The kernels are in fmha_fwd_kernel.h (32x32 MFMAs) and
 // fmha_fwd_kernel16.h (16x16x32 MFMAs).
 #include "fmha_fwd_kernel16p.h"
+#include "fmha_fwd_kernel_ks.h"
 
 namespace cfk {
 namespace {
@@ -32,13 +33,17 @@ using N128_128x128 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 2, 0, tr
 // ... and with the hand-scheduled main loop (key length a multiple of 256, at least 512)
 using A128_256x128 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 2, 0, true, true>;
 
+// ... and for small grids: 32 query rows per workgroup, the eight waves split the keys (fmha_fwd_kernel_ks.h)
+using K64_32x64 = KsCfg<64, 8>;
+using K128_32x64 = KsCfg<128, 8>;
+
 // builds that also write the score tap (debug): 128-row tile only
 using C64Tap = FmhaCfg<64, 64, 4, 2, false, false, false, true>;
 using C128Tap = FmhaCfg<128, 64, 4, 2, false, false, false, true>;
 using C256Tap = FmhaCfg<256, 32, 4, 1, false, false, false, true>;
 
-using All64 = CfgList<C64_128x64, N64_128x64, C64_256x64, C64_128x128, C64_256x128>;
-using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128, N128_128x128, A128_256x128, N128_256x128>;
+using All64 = CfgList<C64_128x64, N64_128x64, C64_256x64, C64_128x128, C64_256x128, K64_32x64>;
+using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128, N128_128x128, A128_256x128, N128_256x128, K128_32x64>;
 
 template <class F>
 bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
@@ -51,8 +56,8 @@ bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
     }
   }
   switch (head_dim) {
-    case 64: select_tile<All64, CfgList<N64_128x64, C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
-    case 128: select_tile<All128, CfgList<A128_256x128, N128_256x128, N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
+    case 64: select_tile<All64, CfgList<K64_32x64, N64_128x64, C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
+    case 128: select_tile<All128, CfgList<K128_32x64, A128_256x128, N128_256x128, N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
     default: return false;
   }
 }

@@ -75,6 +75,7 @@ struct FmhaCfg {
   static constexpr int D = D_, BN = BN_, NWAVES = NWAVES_;
   static constexpr bool M16 = M16_;                             // the fp16 kernel on 16x16x32 MFMAs (fmha_fwd_kernel16.h)
   static constexpr bool ASM = ASM_;                             // ... with the hand-scheduled main loop (gen_fmha_loop16.py)
+  static constexpr bool KSPLIT = false;                         // (true in KsCfg, fmha_fwd_kernel_ks.h: the waves split the keys)
   static constexpr int SUB = SUB_;                              // BN-key sub-tiles per barrier (1 or 2)
   static constexpr int KPRE = KPRE_;                            // K fragments of the next step read before the barrier
   static constexpr int NSLOT = KPRE ? 4 : 2 * SUB;              // LDS slots of one BN-key sub-tile of K
@@ -711,11 +712,14 @@ template <class C>
 __global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(2, 2))) fmha_fwd_kernel16p(const FmhaArgs a);
 template <class C>
 __global__ void __launch_bounds__(C::T) __attribute__((amdgpu_waves_per_eu(2, 2))) fmha_fwd_kernel8p(const FmhaArgs a);
+template <class C>
+__global__ void __launch_bounds__(C::T) fmha_fwd_kernel_ks(const FmhaArgs a);
 
 // the kernel an instantiation runs
 template <class C>
 constexpr auto fmha_kernel_of() {
-  if constexpr (C::ASM && C::QK8) return &fmha_fwd_kernel8p<C>;
+  if constexpr (C::KSPLIT) return &fmha_fwd_kernel_ks<C>;
+  else if constexpr (C::ASM && C::QK8) return &fmha_fwd_kernel8p<C>;
   else if constexpr (C::ASM) return &fmha_fwd_kernel16p<C>;
   else if constexpr (C::M16) return &fmha_fwd_kernel16<C>;
   else return &fmha_fwd_kernel<C>;
@@ -760,6 +764,10 @@ void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
   p->lds_bytes = C::LDS_BYTES;
   p->threads = C::T;
   p->grid = bh * (sq / C::BM);
+  if constexpr (C::KSPLIT) {
+    snprintf(p->kernel, sizeof p->kernel, "fmha_fwd_kernel_ks<%d,%d>", C::D, C::NWAVES);
+    return;
+  }
   snprintf(p->kernel, sizeof p->kernel, "%s<%d,%d,%d,%d,%d,%d,%d,%d,%d,%d,%d,%d>",
            C::ASM ? (C::QK8 ? "fmha_fwd_kernel8p" : "fmha_fwd_kernel16p") : C::M16 ? "fmha_fwd_kernel16" : "fmha_fwd_kernel", C::D, C::BN, C::NWAVES, C::WPE,
            (int)C::QK8, (int)C::PV8, (int)C::VT, (int)C::TAP_S, C::SUB, C::KPRE, (int)C::M16, (int)C::ASM);
@@ -767,9 +775,9 @@ void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
 
 // ---- tile selection.  The reference fixes its tile at compile time (-DQBLKSIZE / -DKBLKSIZE,
 // src/fmha-pipeline/shared_storage.h:4-15, swept by compile_run_all_config.sh:3-6); here every shape is built and one is
-// picked per call.  CFK_FMHA_TILE=<query rows>x<keys>[/16|/16h|/32] (e.g. 256x128, or 256x64/16 for the build on
-// 16x16x32 MFMAs, 256x128/16h for the one with the hand-scheduled main loop), or small | large for the query rows
-// alone, states a wish; a wish no instantiation can serve for the given shape is ignored.  CFK_FMHA_HANDLOOP=0 keeps
+// picked per call.  CFK_FMHA_TILE=<query rows>x<keys>[/16|/16h|/32|/32h] (e.g. 256x128, or 256x64/16 for the build on
+// 16x16x32 MFMAs, 256x128/16h and 256x128/32h for the fp16 / e4m3 ones with the hand-scheduled main loop, 32x64 for the
+// key-split build), or small | large for the query rows alone, states a wish; a wish no instantiation can serve for the given shape is ignored.  CFK_FMHA_HANDLOOP=0 keeps
 // the automatic choice off the hand-scheduled builds (for A/B measurements).
 struct TileWish {
   int bm, bn;  // 0 = no wish
@@ -811,14 +819,15 @@ constexpr bool fits(int sq, int skv) {
 
 // Calls f with the first instantiation of the list that fits the shape and the wish.  Without a wish for the query
 // rows, tiles above 128 rows and the 16x16x32 builds (slower where launch and prologue dominate) are only taken for
-// `big` problems (enough workgroups to fill 256 CUs twice).
+// big problems (size 2: enough workgroups to fill 256 CUs twice), and the key-split build only for small ones (size 0:
+// its 32-row workgroups fit on the chip all at once).
 template <class F, class... Cs>
-bool first_fit(CfgList<Cs...>, int sq, int skv, bool big, TileWish w, F &&f) {
+bool first_fit(CfgList<Cs...>, int sq, int skv, int size, TileWish w, F &&f) {
   bool done = false;
   auto try_one = [&](auto c) {
     using C = decltype(c);
     if (done || !fits<C>(sq, skv)) return;
-    if (w.bm ? C::BM != w.bm : ((C::BM > 128 || C::M16) && !big)) return;
+    if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : ((C::BM > 128 || C::M16) && size != 2))) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
     if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;
     if (w.hand && C::ASM != (w.hand > 0)) return;
@@ -834,11 +843,15 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, bool big, TileWish w, F &&f) {
 template <class All, class Auto, class Fallback, class F>
 void select_tile(int sq, int skv, int bh, F &&f) {
   const bool big = sq % 256 == 0 && (long long)bh * (sq / 256) >= 512;
+  const bool small = (long long)bh * ((sq + 31) / 32) <= 256 && skv >= 128;
+  const int size = big ? 2 : small ? 0 : 1;
   const TileWish w = tile_wish();
-  if ((w.bm || w.bn) && first_fit(All{}, sq, skv, big, w, f)) return;
+  if ((w.bm || w.bn) && first_fit(All{}, sq, skv, size, w, f)) return;
   static const bool no_hand = [] { const char *e = getenv("CFK_FMHA_HANDLOOP"); return e && e[0] == '0'; }();
   // (the hand-scheduled build is a two-pass kernel: not for callers that asked for a data-independent run time)
-  if (first_fit(Auto{}, sq, skv, big, TileWish{0, 0, 0, no_hand || predictable_latency() ? -1 : 0}, f)) return;
+  if (first_fit(Auto{}, sq, skv, size, TileWish{0, 0, 0, no_hand || predictable_latency() ? -1 : 0}, f)) return;
+  // query lengths that only the 32-row (key-split) build divides
+  if (first_fit(Auto{}, sq, skv, 0, TileWish{32, 0, 0, 0}, f)) return;
   f(Fallback{});
 }
 

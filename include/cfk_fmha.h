@@ -58,7 +58,8 @@ typedef struct cfk_fmha_fwd_params {
                         without -DGEMM2FP8 (fmha_forward.cu:446-450)                                            */
   int32_t batch;     /* BATCH                                                                                 */
   int32_t heads;     /* NUMHEADS                                                                              */
-  int32_t seqlen_q;  /* SEQLEN: multiple of 128 (the query rows of a workgroup: 128 or 256)                   */
+  int32_t seqlen_q;  /* SEQLEN: multiple of 128 (the query rows of a workgroup: 128 or 256); fp16 at head dims 64
+                        and 128: multiple of 32 (the small-grid build, 32 rows per workgroup)                  */
   int32_t seqlen_kv; /* KEYLEN: multiple of 64 (32 for fp16 V at head_dim 256); cfk_fmha_forward_plan reports the
                         key tile actually chosen                                                              */
   int32_t head_dim;  /* HEADDIM: 64, 128 or 256 (fmha_forward.cu:746-761)                                     */
@@ -98,10 +99,12 @@ int cfk_fmha_forward_plan(const cfk_fmha_fwd_params *params, int32_t *block_m, i
                           int32_t *lds_bytes, int32_t *threads);
 
 /* The MFMA shape of the kernel build the library would pick for `params`: 32 (32x32x16 / 32x32x64 MFMAs) or 16
- * (16x16x32; fp16 operands, big problems at head dims 64 and 128: the more power-efficient shape on this board).  No
+ * (16x16x32; fp16 operands at head dims 64 and 128, big problems -- the more power-efficient shape on this board -- and
+ * small ones, whose 32-row workgroups split the keys over their waves).  No
  * counterpart in the reference, whose MMA atom is fixed at compile time (src/fmha-pipeline/ss_helper.h:3-94).  The
  * environment variable CFK_FMHA_TILE=<query rows>x<keys>[/16|/16h|/32] overrides the automatic choice of tile and shape
- * (16h: the 16x16x32 build with the hand-scheduled main loop and persistent workgroups, fp16 head dim 128).
+ * (16h / 32h: the builds with the hand-scheduled main loop and persistent workgroups, fp16 / e4m3 at head dim 128; 32x64:
+ * the small-grid build).
  * Does not touch the GPU. */
 int cfk_fmha_forward_mfma(const cfk_fmha_fwd_params *params, int32_t *mfma_rows);
 

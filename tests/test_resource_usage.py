@@ -23,6 +23,9 @@ AUTO_PICKED = {
     "fmha_fwd_kernel<128,64,8,2,0,0,0,0,1,4,0,0>": (0, ""),
     "fmha_fwd_kernel<128,64,8,2,0,0,0,0,1,0,0,0>": (0, ""),
     "fmha_fwd_kernel<128,64,4,2,0,0,0,0,1,0,0,0>": (0, ""),
+    # fp16, small grids (the waves split the keys)
+    "fmha_fwd_kernel_ks<64,8>": (0, ""),
+    "fmha_fwd_kernel_ks<128,8>": (0, ""),
     # fp16 head dim 64
     "fmha_fwd_kernel16<64,64,4,3,0,0,0,0,1,0,1,0>": (14, "the slow path of the row-sum test"),
     "fmha_fwd_kernel<64,64,4,3,0,0,0,0,1,0,0,0>": (0, ""),

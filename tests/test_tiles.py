@@ -36,6 +36,10 @@ CASES = {
     # the e4m3 build with the hand-scheduled loop and persistent workgroups (key length a multiple of 256, from 4096): the
     # scheduled loop, 4352 keys (an odd number of loop turns), 2x10 heads x 4096 rows = 320 items (a quarter of the
     # workgroups take a second one), climbing keys (the vote, the max-tracking loop, then a next item: 5x13x1024 rows = 260)
+    # 32 query rows per workgroup, the eight waves split the keys (the automatic choice for small grids): key lengths with
+    # fewer tiles than waves, with tiles left over, query lengths that no other tile divides, taps, climbing keys
+    "32x64": ["f16:1,512,8,64", "f16:1,512,2,128", "f16:2,96,3,64,64", "f16:1,160,2,128,192", "f16:1,128,2,64,1216", "f16nt:1,256,2,128,640",
+              "f16climb:1,256,2,64,512", "f16climb:1,128,2,128,1024", "f16:3,2048,4,128,2048"],
     "256x128/32h": ["f8:1,256,2,128,4096", "f8:1,512,1,128,4352", "f8:2,4096,10,128", "f8climb:1,256,2,128,4096", "f8climb:5,1024,13,128,4096"],
 }
 
@@ -44,23 +48,27 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     # the plan query needs no GPU; a wish no instantiation serves is ignored
     f = pkg.fmha
     code = ("import sys; sys.path.insert(0, %r); import __graft_entry__ as e; p = e.load_package(); f = p.fmha; "
-            "print(f.fmha_forward_plan(f.CFK_FP16, 2, 4, 512, 512, 128)[:2], f.fmha_forward_plan(f.CFK_FP16, 2, 4, 512, 512, 256)[:2], "
-            "f.fmha_forward_plan(f.CFK_FP8_E4M3, 2, 4, 512, 512, 128)[:2], f.fmha_forward_plan(f.CFK_FP16, 2, 4, 384, 384, 128)[:2])" % ROOT)
+            "print(f.fmha_forward_plan(f.CFK_FP16, 2, 4, 1536, 512, 128)[:2], f.fmha_forward_plan(f.CFK_FP16, 2, 4, 1536, 512, 256)[:2], "
+            "f.fmha_forward_plan(f.CFK_FP8_E4M3, 2, 4, 1536, 512, 128)[:2], f.fmha_forward_plan(f.CFK_FP16, 2, 16, 384, 384, 128)[:2], "
+            "f.fmha_forward_plan(f.CFK_FP16, 2, 4, 512, 512, 128)[:2])" % ROOT)
     def plans(wish):
         env = dict(os.environ)
         env.pop("CFK_FMHA_TILE", None)
         if wish:
             env["CFK_FMHA_TILE"] = wish
         return subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout.strip()
-    assert plans(None) == "(128, 64) (128, 32) (128, 64) (128, 64)"           # small problems: 128-row tiles
-    assert plans("256x128") == "(256, 128) (128, 32) (256, 128) (128, 64)"     # no such tile at head dim 256; 384 % 256 != 0
-    assert plans("large") == "(256, 64) (128, 32) (256, 64) (128, 64)"
-    assert plans("128x128") == "(128, 128) (128, 32) (128, 128) (128, 128)"
+    # medium problems: 128-row tiles; small ones (the last: 128 workgroups of 32 rows fit on the chip at once): fp16 at head
+    # dims 64 and 128 takes 32-row workgroups whose waves split the keys
+    assert plans(None) == "(128, 64) (128, 32) (128, 64) (128, 64) (32, 64)"
+    assert plans("256x128") == "(256, 128) (128, 32) (256, 128) (128, 64) (256, 128)"     # no such tile at head dim 256; 384 % 256 != 0
+    assert plans("large") == "(256, 64) (128, 32) (256, 64) (128, 64) (256, 64)"
+    assert plans("128x128") == "(128, 128) (128, 32) (128, 128) (128, 128) (128, 128)"
+    assert plans("32x64") == "(32, 64) (128, 32) (128, 64) (32, 64) (32, 64)"              # fp16 at head dims 64 / 128 only
     # the MFMA shape suffix: served for fp16 at head dims 64/128 only (e4m3 and head dim 256 ignore the wish)
     mfma_code = ("import sys; sys.path.insert(0, %r); import __graft_entry__ as e; p = e.load_package(); f = p.fmha; "
-                 "print(f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 512, 512, 128), f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 512, 512, 64), "
-                 "f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 512, 512, 256), f.fmha_forward_mfma(f.CFK_FP8_E4M3, 2, 4, 512, 512, 128), "
-                 "f.fmha_forward_plan(f.CFK_FP16, 2, 4, 512, 512, 128)[:2])" % ROOT)
+                 "print(f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 128), f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 64), "
+                 "f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 256), f.fmha_forward_mfma(f.CFK_FP8_E4M3, 2, 4, 1536, 512, 128), "
+                 "f.fmha_forward_plan(f.CFK_FP16, 2, 4, 1536, 512, 128)[:2])" % ROOT)
     def shapes(wish):
         env = dict(os.environ, CFK_FMHA_TILE=wish)
         return subprocess.run([sys.executable, "-c", mfma_code], env=env, capture_output=True, text=True, check=True).stdout.strip()
@@ -73,7 +81,7 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     assert shapes("256x128/16h") == "16 32 32 32 (256, 128)"  # ... with the hand-scheduled loop
     # the hand-scheduled build needs 160 KB of LDS; a wish for the compiler-scheduled one (no `h`) is kept apart from it
     lds_code = ("import sys; sys.path.insert(0, %r); import __graft_entry__ as e; p = e.load_package(); f = p.fmha; "
-                "print(f.fmha_forward_plan(f.CFK_FP16, 2, 4, 512, 512, 128)[2], f.fmha_forward_plan(f.CFK_FP16, 2, 4, 512, 384, 128)[:3])" % ROOT)
+                "print(f.fmha_forward_plan(f.CFK_FP16, 2, 4, 1536, 512, 128)[2], f.fmha_forward_plan(f.CFK_FP16, 2, 4, 1536, 384, 128)[:3])" % ROOT)
     def lds(wish):
         env = dict(os.environ, CFK_FMHA_TILE=wish)
         return subprocess.run([sys.executable, "-c", lds_code], env=env, capture_output=True, text=True, check=True).stdout.strip()
@@ -85,7 +93,10 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     assert f.fmha_forward_mfma(f.CFK_FP16, 8, 16, 2048, 2048, 128) == 16
     assert f.fmha_forward_mfma(f.CFK_FP16, 4, 32, 4096, 4096, 64) == 16
     assert f.fmha_forward_plan(f.CFK_FP16, 4, 32, 4096, 4096, 64)[:2] == (128, 64)
-    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 512, 512, 128) == 32
+    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 128) == 32
+    assert f.fmha_forward_kernel(f.CFK_FP16, 1, 8, 512, 512, 64) == "fmha_fwd_kernel_ks<64,8>"      # benchmark configuration 1
+    assert f.fmha_forward_kernel(f.CFK_FP16, 2, 4, 512, 512, 128) == "fmha_fwd_kernel_ks<128,8>"
+    assert f.fmha_forward_plan(f.CFK_FP16, 1, 2, 96, 192, 64)[:2] == (32, 64)                       # query rows a multiple of 32
     assert f.fmha_forward_mfma(f.CFK_FP16, 2, 8, 8192, 8192, 256) == 32
     assert f.fmha_forward_mfma(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128) == 32
     assert f.fmha_forward_plan(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128)[:2] == (256, 128)
@@ -107,7 +118,7 @@ def test_forced_tiles_match_the_oracle(wish):
         print(row)
         assert (row["block_m"], row["block_n"]) == (bm, bn), row     # the wished tile really ran
         if row["case"].startswith("f16"):
-            assert row["mfma"] == int(mfma or 32), row               # ... on the wished MFMA shape
+            assert row["mfma"] == (16 if bm == 32 else int(mfma or 32)), row   # ... on the wished MFMA shape (the 32-row build: 16x16x32)
             # row-max tap (relative to the largest row max): exact fp32 products, so only summation order separates
             # it from the oracle; row-sum tap (relative): the kernel adds the weights as rounded to fp16 (2^-11 each,
             # unbiased), the oracle the fp32 values
