@@ -59,6 +59,11 @@ WORKLOADS = {
     "cfg3": dict(kind="fmha", dtype="f16", B=2, H=8, S=8192, D=256, scale=None),
     "cfg4": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None),
     "cfg5": dict(kind="gemm", dtype="f16", M=8192, N=8192, K=8192),
+    # the data-dependent side of the e4m3 kernel: keys whose scores climb along the key axis send every workgroup through
+    # its second (max-tracking) pass; `one_pass` runs the same data under cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, 1)
+    "cfg4_climb": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None, climb=True),
+    "cfg4_climb_one_pass": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None, climb=True, one_pass=True),
+    "cfg4_one_pass": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None, one_pass=True),
     "d64_f16": dict(kind="fmha", dtype="f16", B=4, H=32, S=4096, D=64, scale=None),   # the reference sweep's head size 64
     "d64_f8": dict(kind="fmha", dtype="f8", B=4, H=32, S=4096, D=64, scale=None),
     "gemm_f32": dict(kind="gemm", dtype="f32", M=8192, N=8192, K=8192, max_steps=50),  # the CuTe example's type 1
@@ -69,6 +74,10 @@ NAMES = {
     "cfg3": "fmha_fwd fp16 B=2 H=8 S=8192 D=256 non-causal",
     "cfg4": "fmha_fwd fp8-e4m3 B=4 H=16 S=4096 D=128 non-causal, per-tensor amax scales, V [B,S,H,D]",
     "cfg5": "gemm fp16 M=N=K=8192 TN fp32-accumulate",
+    "cfg4_climb": "fmha_fwd fp8-e4m3 B=4 H=16 S=4096 D=128, keys scaled 1..4 along the key axis and one key x8 (scores climb: "
+                  "every workgroup takes the second, max-tracking pass)",
+    "cfg4_climb_one_pass": "... the same data with cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, 1): max-tracking pass only",
+    "cfg4_one_pass": "fmha_fwd fp8-e4m3 B=4 H=16 S=4096 D=128 N(0,1) data with cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, 1)",
     "d64_f16": "fmha_fwd fp16 B=4 H=32 S=4096 D=64 non-causal (the reference sweep's problem at head size 64)",
     "d64_f8": "fmha_fwd fp8-e4m3 B=4 H=32 S=4096 D=64 non-causal, per-tensor amax scales, V [B,S,H,D]",
     "gemm_f32": "gemm fp32 M=N=K=8192 TN (fp32 MFMA: gfx950 has no tf32)",
@@ -106,6 +115,10 @@ def _make_fmha(pkg, w, seed=3080):
     B, H, S, D = w["B"], w["H"], w["S"], w["D"]
     gens = [torch.Generator(device=dev).manual_seed(seed + i) for i in (1, 2, 3)]
     q, k, v = (torch.randn((B, S, H, D), generator=g, device=dev, dtype=torch.float32) for g in gens)
+    if w.get("climb"):   # (tests/_util.py: climbing_keys with the e4m3 test's parameters)
+        ramp = 1.0 + 3.0 * torch.arange(S, device=dev, dtype=torch.float32) / (S - 1)
+        ramp[(3 * S) // 4 + 3] *= 8.0
+        k = k * ramp[None, :, None, None]
     kw = dict(softmax_scale=w["scale"])
     if w["dtype"] == "f16":
         q, k, v = q.half(), k.half(), v.half()
@@ -137,11 +150,21 @@ def run_workload(pkg, name, steps, warmup):
     # configuration 1 is a 9-microsecond kernel: the reference's protocol (mean over back-to-back launches) needs
     # many more of them for a stable mean
     n = steps * 20 if name == "cfg1" else min(steps, w.get("max_steps", steps))
-    ms, wall_ms = _time_launches(fn, n, warmup)
+    if w.get("one_pass"):
+        pkg.fmha.set_option(pkg.fmha.CFK_OPT_PREDICTABLE_LATENCY, 1)
+    try:
+        kernel = None
+        if w["kind"] == "fmha":   # the instantiation the library launches for this call (cfk_fmha_forward_kernel)
+            f = pkg.fmha
+            kernel = f.fmha_forward_kernel(f.CFK_FP8_E4M3 if w["dtype"] == "f8" else f.CFK_FP16, w["B"], w["H"], w["S"], w["S"], w["D"])
+        ms, wall_ms = _time_launches(fn, n, warmup)
+    finally:
+        if w.get("one_pass"):
+            pkg.fmha.set_option(pkg.fmha.CFK_OPT_PREDICTABLE_LATENCY, 0)
     tflops = flop / (ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[w["dtype"]]
     return dict(workload=NAMES[name], ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, flop_per_step=flop,
-                dtype=w["dtype"], frac_of_peak=tflops / peak, peak_tflops=peak), keep
+                dtype=w["dtype"], frac_of_peak=tflops / peak, peak_tflops=peak, kernel=kernel), keep
 
 
 def cpu_baseline(pkg, w, budget_s=12.0):
@@ -207,7 +230,7 @@ def main():
                 r, keep = run_workload(pkg, name, args.steps, args.warmup)
                 del keep
                 torch.cuda.empty_cache()
-                secondary.append({k: r[k] for k in ("workload", "ms_per_step", "tflops", "dtype", "frac_of_peak")})
+                secondary.append({k: r[k] for k in ("workload", "kernel", "ms_per_step", "tflops", "dtype", "frac_of_peak")})
             except pkg.CfkError as e:
                 secondary.append({"workload": NAMES[name], "error": str(e)})
     w = WORKLOADS[args.workload]
@@ -225,7 +248,7 @@ def main():
         "vs_baseline": None,
         "dtype": w["dtype"],
         "data": "synthetic",
-        "config": {"workload": main_res["workload"], "flop_per_step": main_res["flop_per_step"],
+        "config": {"workload": main_res["workload"], "kernel": main_res["kernel"], "flop_per_step": main_res["flop_per_step"],
                    "layout": "[B,S,H,D]", "seeds": [3081, 3082, 3083],
                    "protocol": "reference protocol (warm-up launches, then the mean of back-to-back launches between two "
                                "events on the launch stream, src/fmha-pipeline/fmha_forward.cu:578-593) preceded by an "
