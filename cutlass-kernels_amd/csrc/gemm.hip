@@ -429,6 +429,13 @@ gemm_kernel16(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B, co
   constexpr int SPM = NBN;                    // slots per m block
   constexpr int ST_EVERY = NB * NBN / CPT;    // a staging piece every so many slots of K-step 0
   static_assert(KS == 2 && ST_EVERY >= 2 && NB * NBN % CPT == 0, "slot layout");
+  // The multiplies are asm statements with "+a" accumulators: the compiler's hazard recognizer does not see the
+  // matrix-pipe write -> accumulate-read dependency between two of them, so the distance between two multiplies into
+  // one accumulator is this layout's business.  Every accumulator block is used once per K-step: NB * NBN multiplies
+  // lie between two uses (64), each holding the pipe for the 4 passes of v_mfma_f32_16x16x32_f16; back-to-back
+  // dependent MFMAs of this shape need 4 passes + 2 wait states.  Fewer blocks per wave than that (or a reordering that
+  // revisits a block within one K-step) would need nops here.
+  static_assert(NB * NBN >= 8, "distance between two multiplies into one accumulator: at least the MFMA's passes plus its wait states");
   Rsrc ga, gb;
   tile_ptrs(0, ga, gb);
 #pragma unroll
