@@ -4,7 +4,7 @@
 // instruction order hides LDS and MFMA latency, and the order that strategy finds is the faster one: 994-1001 against
 // 928 TFLOP/s on B=2 H=8 S=8192 with N(0,1) tensors, 1206 against 1024 with constant tensors.  Every kernel with two or
 // three waves per SIMD loses under it (registers spill), so it is not a library-wide flag.
-#include "fmha_fwd_kernel.h"
+#include "fmha_fwd_kernel16p.h"
 
 namespace cfk {
 namespace {
@@ -17,8 +17,11 @@ using C256_128x32P = FmhaCfg<256, 32, 4, 1, false, false, false, false, 1, 4>;  
 // one: 572 TFLOP/s), and run as fast as 32-key tiles (1003-1007 against 1010-1016 TFLOP/s on B=2 H=8 S=8192, two 32-key
 // tiles per barrier 1010-1013): a choice for the tile sweep, not the automatic one.
 using C256_128x64 = FmhaCfg<256, 64, 4, 1, false, false>;
-using All256 = CfgList<C256_128x32P, C256_128x32, C256_128x64>;
-using Auto256 = CfgList<C256_128x32P, C256_128x32>;
+// The hand-scheduled persistent build on 16x16x32 MFMAs (fmha_fwd_kernel16p.h; key length a multiple of 128, at least
+// 256): two 32-key tiles per barrier, big problems only
+using A256_128x64 = FmhaCfg<256, 32, 4, 1, false, false, false, false, 2, 0, true, true>;
+using All256 = CfgList<C256_128x32P, C256_128x32, C256_128x64, A256_128x64>;
+using Auto256 = CfgList<A256_128x64, C256_128x32P, C256_128x32>;
 
 template <class F>
 void dispatch(int sq, int skv, int bh, F &&f) {

@@ -1,9 +1,13 @@
 #!/usr/bin/env python3
-"""Generator of the hand-scheduled main loop of the fp16 FMHA forward kernel on 16x16x32 MFMAs
-(fmha_fwd_kernel16.h, FmhaCfg::ASM), head dim 128, 256 query rows per workgroup (8 waves x 32 rows, two waves per SIMD).
+"""Generator of the hand-scheduled main loops of the fp16 FMHA forward kernel on 16x16x32 MFMAs (fmha_fwd_kernel16p.h,
+FmhaCfg::ASM), in two shapes:
+  d128  head dim 128, 64-key tiles, 256 query rows per workgroup (8 waves x 32 rows, two waves per SIMD)
+  d256  head dim 256, 32-key tiles, 128 query rows per workgroup (4 waves x 32 rows, one wave per SIMD: Q and O alone
+        are 192 registers per lane; O lives in the accumulation registers a[0:127])
+Both have the same timeline (64 MFMA slots and 16 KB of K and of V per tile); the text below describes d128.
 
-    python3 gen_fmha_loop16.py            # rewrites fmha_fwd_loop16_d128.inc beside this file
-    python3 gen_fmha_loop16.py --check    # exit status 1 if that file is not what the generator produces
+    python3 gen_fmha_loop16.py            # rewrites fmha_fwd_loop16_d128.inc and fmha_fwd_loop16_d256.inc beside this file
+    python3 gen_fmha_loop16.py --check    # exit status 1 if those files are not what the generator produces
 
 Why a generator: the loop is one inline-asm statement of ~2800 instructions with every register assigned by hand.
 Left to the compiler, the step comes out as blocks (all MFMAs of a GEMM, then all of the softmax), the two waves of
@@ -56,23 +60,17 @@ import json
 import os
 import sys
 
-# ---- shape (head dim 128, 64-key tiles, 8 waves) ---------------------------------------------------------------
-D, BN, NWAVES = 128, 64, 8
-KB, KS, DB, PS, QB = BN // 16, D // 32, D // 16, BN // 32, 2
-K_PITCH = V_PITCH = D * 2
-K_TILE = V_TILE = BN * K_PITCH          # 16384
-NSLOT = 4
+# ---- shape --------------------------------------------------------------------------------------------------------
+SHAPE = "d128"
+QB, NSLOT = 2, 4
+K_TILE = V_TILE = 16384                 # both shapes: 64 keys x 256 B = 32 keys x 512 B
 K_ST0, V_ST0 = 0, NSLOT * K_TILE        # LDS map: K slots, then V slots (the read addresses include these bases)
-IPW = 2                                  # copies per wave and tile (K and V alike)
 
 # ---- how the row sum l is taken ----------------------------------------------------------------------------------
 #   "mfma": l += 1 . P on the matrix pipe (sums P as rounded to fp16, the weights the second GEMM applies)
 #   "add":  v_add_f32 over the fp32 weights before the cast (online_softmax.h:173-206), two chains per query block
 #   "dot":  v_dot2c_f32_f16 over the rounded weights, summed per tile in the order of fmha_fwd_kernel16.h's loop
 ROWSUM = "add"
-# ---- registers ---------------------------------------------------------------------------------------------------
-O0, SA0, SB0, Q0, P0, RING0 = 192, 128, 160, 96, 80, 48
-KRD0, VRD0, GOK0, GOV0 = 24, 28, 36, 38
 RING = 8
 LOOKAHEAD = 7      # fragments requested ahead of use
 HOLD = 4           # MFMAs of a super-step issued behind its barrier
@@ -83,9 +81,20 @@ ABLATE = set(os.environ.get("LOOP16_ABLATE", "").split(",")) - {""}
 
 
 def configure():
-    """derived constants; call again after changing ROWSUM or a parameter"""
+    """derived constants; call again after changing SHAPE, ROWSUM or a parameter"""
     g = globals()
-    if ROWSUM == "mfma":
+    if SHAPE == "d128":
+        g.update(D=128, BN=64, NWAVES=8, O_ACC=False, O0=192, SA0=128, SB0=160, Q0=96, P0=80, RING0=48, KRD0=24, VRD0=28, GOK0=36, GOV0=38)
+    else:
+        assert ROWSUM == "add"
+        g.update(D=256, BN=32, NWAVES=4, O_ACC=True, O0=0, SA0=224, SB0=240, Q0=160, P0=144, RING0=112, KRD0=96, VRD0=80, GOK0=72, GOV0=76)
+    g.update(KB=BN // 16, KS=D // 32, DB=D // 16, PS=BN // 32, K_PITCH=2 * D, V_PITCH=2 * D)
+    g["IPW"] = K_TILE // 1024 // NWAVES     # copies per wave and tile (K and V alike)
+    g["QKS"] = KS * KB * QB                 # MFMA slots of S = K.Q^T
+    if SHAPE == "d256":
+        g.update(M0R=70, LA0=64, QOFF0=68, LOW=64, L_OUT=(64, 66), T=64, L_TOTAL=False)
+        start = 36   # S(t+1) is complete at slot 32; P(t+1) has to be before slot 32 of the next period
+    elif ROWSUM == "mfma":
         g.update(M0R=18, ONES0=20, LACC0=40, QOFF0=16, LOW=16, L_OUT=(40, 44), T=68, L_TOTAL=True)
         start = 46
     elif ROWSUM == "add":
@@ -94,15 +103,19 @@ def configure():
     else:
         g.update(M0R=40, L0=42, RS0=44, RS20=46, QOFF0=22, LOW=22, L_OUT=(42, 43), T=64, L_TOTAL=False)
         start = 44
-    g["PV0"] = [32 + ps * (16 + (2 if ROWSUM == "mfma" else 0)) for ps in range(PS)]   # first slot of each key half's P.V
+    g["PV0"] = [QKS + ps * (DB * QB + (2 if ROWSUM == "mfma" else 0)) for ps in range(PS)]   # first slot of each key half's P.V
     g["V_START"] = start if VALU_START is None else VALU_START
-    g["V_RATE"] = sum(c for _, c in softmax_ops(0)) / float(T) if VALU_RATE is None else VALU_RATE
+    span = T if PS == 2 else T - 6   # one key half per tile: the whole of P is needed at once, by the first P.V slot
+    g["V_RATE"] = sum(c for _, c in softmax_ops(0)) / float(span) if VALU_RATE is None else VALU_RATE
 
 
 def o_reg(db, qb): return O0 + 4 * (2 * db + qb)
+def o_txt(db, qb): return ("a[%d:%d]" if O_ACC else "v[%d:%d]") % (o_reg(db, qb), o_reg(db, qb) + 3)
 def s_reg(t, kb, qb): return (SA0 if t % 2 == 0 else SB0) + 4 * (2 * kb + qb)
-def q_reg(qb, s): return Q0 + 4 * (4 * qb + s)
-def p_reg(qb, ps): return P0 + 4 * (2 * qb + ps)
+def q_reg(qb, s): return Q0 + 4 * (KS * qb + s)
+def p_reg(t, qb, ps):
+    # one key half per tile (d256): P is double-buffered by tile parity, its softmax runs beside the other set's P.V
+    return P0 + (8 * (t % 2) + 4 * qb if PS == 1 else 4 * (2 * qb + ps))
 def vr(r, n=4): return "v[%d:%d]" % (r, r + n - 1)
 
 
@@ -124,13 +137,13 @@ class Frag:
         if self.kind == 'K':
             d = s_reg(self.t, self.b, qb)
             return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (vr(d), vr(self.reg), vr(q_reg(qb, self.a)), "0" if self.a == 0 else vr(d))
-        d = o_reg(self.b, qb)
-        return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (vr(d), vr(self.reg), vr(p_reg(qb, self.a)), vr(d))
+        d = o_txt(self.b, qb)
+        return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (d, vr(self.reg), vr(p_reg(self.t, qb, self.a)), d)
 
 
-def sum_mfma(ps, qb):
+def sum_mfma(t, ps, qb):
     d = LACC0 + 4 * qb
-    return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (vr(d), vr(ONES0), vr(p_reg(qb, ps)), vr(d))
+    return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (vr(d), vr(ONES0), vr(p_reg(t, qb, ps)), vr(d))
 
 
 def softmax_ops(t):
@@ -139,7 +152,7 @@ def softmax_ops(t):
     for kb in range(KB):
         for qb in range(QB):
             s = s_reg(t, kb, qb)
-            p = p_reg(qb, kb // 2) + 2 * (kb % 2)
+            p = p_reg(t, qb, kb // 2) + 2 * (kb % 2)
             for i in range(4): ops.append(("v_fma_f32 v%d, v%d, %%[c], -v%d" % (s + i, s + i, M0R + qb), 1))
             for i in range(4): ops.append(("v_exp_f32 v%d, v%d" % (s + i, s + i), 2))
             if ROWSUM == "add" and "rowsum" not in ABLATE:
@@ -199,7 +212,7 @@ def schedule(n_tiles):
                 f = Frag('V', t, ps, db, base + PV0[ps] + 2 * db, len(frags)); frags.append(f)
                 for qb in range(QB): slot_item[f.slot0 + qb] = (f, qb)
             if ROWSUM == "mfma":
-                for qb in range(QB): slot_item[base + PV0[ps] + 2 * DB + qb] = ("L", ps, qb)
+                for qb in range(QB): slot_item[base + PV0[ps] + 2 * DB + qb] = ("L", t, ps, qb)
     # ---- vector work: slot -> [text]; positions before slot 0 are issued ahead of it
     valu_at = {}
     for t in range(n_tiles):
@@ -230,7 +243,7 @@ def schedule(n_tiles):
     for i, grp in enumerate(groups): copies_at[Z + 1 + 4 * i] = grp
     for i in range(QB * KS):
         qb, ks = i // KS, i % KS
-        copies_at.setdefault(Z + 33 + 3 * i, []).append("global_load_dwordx4 %s, v%d, %%[qn] offset:%d" % (vr(q_reg(qb, ks)), QOFF0 + qb, 64 * ks))
+        copies_at.setdefault(Z + QKS + 1 + 3 * i, []).append("global_load_dwordx4 %s, v%d, %%[qn] offset:%d" % (vr(q_reg(qb, ks)), QOFF0 + qb, 64 * ks))
     # ---- emission
     segs, cur = [], []
     nread = 0             # LDS read instructions issued so far
@@ -259,7 +272,7 @@ def schedule(n_tiles):
     # ahead of slot 0: first operand requests, then the vector work that precedes the timeline
     cur.append("s_waitcnt lgkmcnt(0)")
     cur.append("s_nop 7"); cur.append("s_nop 7")   # MFMA results of the caller's S(0) are read by vector instructions
-    for r in range(O0, O0 + 64): cur.append("v_mov_b32 v%d, 0" % r)
+    for r in range(O0, O0 + 4 * DB * QB): cur.append(("v_accvgpr_write_b32 a%d, 0" if O_ACC else "v_mov_b32 v%d, 0") % r)
     if ROWSUM == "mfma":
         for r in range(ONES0, ONES0 + 4): cur.append("v_mov_b32 v%d, 0x3c003c00" % r)
         for r in range(LACC0, LACC0 + 8): cur.append("v_mov_b32 v%d, 0" % r)
@@ -281,7 +294,7 @@ def schedule(n_tiles):
         it = slot_item[slot]
         if it is not None and "mfma" not in ABLATE:
             if it[0] == "L":
-                cur.append(sum_mfma(it[1], it[2]))
+                cur.append(sum_mfma(it[1], it[2], it[3]))
             else:
                 f, qb = it
                 if qb == 0 and read_end[f.idx] > done_reads:
@@ -325,16 +338,16 @@ def program(n_tiles):
 
 def render():
     """the C++ text of the include: a flag the caller needs, then the complete asm statement.  It expects these names
-    in scope: f32x16 o0..o3 (out), sa0, sa1 (in, clobbered), q0v, q1v (in: this item's Q; out: the next item's); float
-    l0, l1 (out); uint64_t kptr, vptr (in: this item's K tile 3 / V tile 2; out: the same of the next item), kn, vn, qn
-    (the next item's K, V and this wave's Q rows); uint32_t nloop, k_rd[4], v_rd[8], goff_k[2], goff_v[2], qoff[2],
-    lds_wave, tile_stride; float m_ref[2], c_log2."""
+    in scope: bool sum_is_complete (out: the flag), f32x16 o0, o1, .. (out: the O accumulators, 16 registers each, in register order), sa0, .. (in, clobbered:
+    S(0)), q0, .. (in: this item's Q; out: the next item's); float l0, l1 (out); uint64_t kptr, vptr (in: this item's K
+    tile 3 / V tile 2; out: the same of the next item), kn, vn, qn (the next item's K, V and this wave's Q rows);
+    uint32_t nloop, k_rd[KS], v_rd[DB], goff_k[IPW], goff_v[IPW], qoff[2], lds_wave, tile_stride; float m_ref[2], c_log2."""
     head, body, tail = folded()
     L = []
-    L.append("// GENERATED by gen_fmha_loop16.py -- do not edit.  The hand-scheduled main loop of fmha_fwd_kernel16 (FmhaCfg::ASM: head")
-    L.append("// dim 128, 256 x 128): %d + %d (loop) + %d instructions, row sum by \"%s\"." % (len(head), len(body), len(tail), ROWSUM))
+    L.append("// GENERATED by gen_fmha_loop16.py -- do not edit.  The hand-scheduled main loop of fmha_fwd_kernel16p (FmhaCfg::ASM: head")
+    L.append("// dim %d, %d x %d): %d + %d (loop) + %d instructions, row sum by \"%s\"." % (D, 32 * NWAVES, 2 * BN, len(head), len(body), len(tail), ROWSUM))
     L.append("// l0 / l1 hold the complete row sum of the lane's query in every lane (true) or the lane's share of it (false)")
-    L.append("constexpr bool kLoop16SumIsComplete = %s;" % ("true" if L_TOTAL else "false"))
+    L.append("sum_is_complete = %s;" % ("true" if L_TOTAL else "false"))
     L.append("asm volatile(")
     def emit(ins): L.append('    "%s\\n"' % ins)
     for i in head: emit(i)
@@ -347,9 +360,13 @@ def render():
     emit("s_cbranch_scc1 1b")
     emit("2:")
     for i in tail: emit(i)
-    used = set(range(O0, O0 + 64)) | set(range(SA0, SA0 + 32)) | set(range(Q0, Q0 + 32)) | set(range(KRD0, GOV0 + 2)) | {M0R, M0R + 1, QOFF0, QOFF0 + 1} | set(L_OUT)
-    L.append('    : "={v[192:207]}"(o0), "={v[208:223]}"(o1), "={v[224:239]}"(o2), "={v[240:255]}"(o3), "={v%d}"(l0), "={v%d}"(l1),' % L_OUT)
-    L.append('      "+{v[128:143]}"(sa0), "+{v[144:159]}"(sa1), "+{v[96:111]}"(q0v), "+{v[112:127]}"(q1v), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), [nloop] "+s"(nloop)')
+    def vec16(base, name, n, kind="v", mode="="):
+        return ['"%s{%s[%d:%d]}"(%s%d)' % (mode, kind, base + 16 * i, base + 16 * i + 15, name, i) for i in range(n)]
+    n_o, n_s, n_q = 4 * DB * QB // 16, 4 * KB * QB // 16, 4 * KS * QB // 16
+    outs = vec16(O0, "o", n_o, "a" if O_ACC else "v") + ['"={v%d}"(l0)' % L_OUT[0], '"={v%d}"(l1)' % L_OUT[1]]
+    inouts = vec16(SA0, "sa", n_s, mode="+") + vec16(Q0, "q", n_q, mode="+") + ['"+{s[40:41]}"(kptr)', '"+{s[42:43]}"(vptr)', '[nloop] "+s"(nloop)']
+    L.append("    : " + ", ".join(outs) + ",")
+    L.append("      " + ", ".join(inouts))
     ins = ['"{v%d}"(qoff[%d])' % (QOFF0 + i, i) for i in range(QB)] + ['[kn] "s"(kn)', '[vn] "s"(vn)', '[qn] "s"(qn)']
     ins += ['"{v%d}"(k_rd[%d])' % (KRD0 + i, i) for i in range(KS)] + ['"{v%d}"(v_rd[%d])' % (VRD0 + i, i) for i in range(DB)]
     ins += ['"{v%d}"(goff_k[%d])' % (GOK0 + i, i) for i in range(IPW)] + ['"{v%d}"(goff_v[%d])' % (GOV0 + i, i) for i in range(IPW)]
@@ -357,6 +374,9 @@ def render():
     ins += ['[c] "s"(c_log2)', '[ldsw] "s"(lds_wave)', '[stride] "s"(tile_stride)']
     if ROWSUM == "dot": ins.append('[ones] "s"(0x3c003c00u)')
     L.append("    : " + ", ".join(ins))
+    used = set(range(SA0, SA0 + 16 * n_s)) | set(range(Q0, Q0 + 16 * n_q)) | set(range(KRD0, KRD0 + KS)) | set(range(VRD0, VRD0 + DB))
+    used |= set(range(GOK0, GOK0 + IPW)) | set(range(GOV0, GOV0 + IPW)) | {M0R, M0R + 1, QOFF0, QOFF0 + 1} | set(L_OUT)
+    if not O_ACC: used |= set(range(O0, O0 + 16 * n_o))
     clob = ['"memory"', '"scc"', '"m0"'] + ['"v%d"' % r for r in range(LOW, 256) if r not in used]
     L.append("    : " + ", ".join(clob) + ");")
     return "\n".join(L) + "\n"
@@ -364,11 +384,17 @@ def render():
 
 configure()
 if __name__ == "__main__":
-    for k, v in json.loads(os.environ.get("LOOP16_SET", "{}")).items(): globals()[k] = v
-    configure()
-    out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fmha_fwd_loop16_d128.inc")
-    txt = render()
-    if "--check" in sys.argv:
-        sys.exit(0 if os.path.exists(out) and open(out).read() == txt else 1)
-    open(out, "w").write(txt)
-    print("wrote", out, len(txt.splitlines()), "lines")
+    overrides = json.loads(os.environ.get("LOOP16_SET", "{}"))
+    stale = False
+    for shape in ("d128", "d256"):
+        SHAPE = shape
+        for k, v in overrides.items(): globals()[k] = v
+        configure()
+        out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fmha_fwd_loop16_%s.inc" % shape)
+        txt = render()
+        if "--check" in sys.argv:
+            stale = stale or not (os.path.exists(out) and open(out).read() == txt)
+        else:
+            open(out, "w").write(txt)
+            print("wrote", out, len(txt.splitlines()), "lines")
+    sys.exit(1 if stale else 0)

@@ -1,6 +1,7 @@
-"""Symbolic check of the hand-scheduled main loop of the fp16 kernel (cutlass-kernels_amd/csrc/gen_fmha_loop16.py).
+"""Symbolic check of the hand-scheduled main loops of the fp16 kernel (cutlass-kernels_amd/csrc/gen_fmha_loop16.py), in
+both of its shapes (head dim 128: 8 waves, 64-key tiles; head dim 256: 4 waves, 32-key tiles, O in accumulation registers).
 
-The loop is ~2800 hand-allocated instructions inside one asm statement, where neither the compiler's register
+A loop is ~2800 hand-allocated instructions inside one asm statement, where neither the compiler's register
 allocator nor its hazard recognizer helps.  This test walks the instruction text a wave executes (loop unrolled for
 several key lengths) with symbolic register contents and checks, instruction by instruction:
   * every MFMA multiplies the operands the algorithm wants (K fragment x Q of the same K-step into the right score
@@ -101,7 +102,10 @@ class Checker:
     # ---- instructions
     def run(self, prog):
         g = self.g
-        R = lambda s: [int(x) for x in re.match(r"v\[(\d+):(\d+)\]", s).groups()]
+        def R(s):   # register range -> [first, last]; accumulation registers a[n] are numbered 1000 + n
+            m = re.match(r"([va])\[(\d+):(\d+)\]", s)
+            base = 1000 if m.group(1) == "a" else 0
+            return [base + int(m.group(2)), base + int(m.group(3))]
         for ins in prog:
             self.cur = ins
             op, _, rest = ins.partition(" ")
@@ -126,14 +130,17 @@ class Checker:
             elif op == "v_mov_b32":
                 assert a[1] in ("0", "0x3c003c00")
                 self.put(int(a[0][1:]), ("zero",) if a[1] == "0" else ("one",), 10 ** 9, "valu")
+            elif op == "v_accvgpr_write_b32":
+                assert a[1] == "0" and a[0][0] == "a"
+                self.put(1000 + int(a[0][1:]), ("zero",), 10 ** 9, "valu")
             elif op == "ds_read_b128":
                 lo, hi = R(a[0])
                 assert hi == lo + 3 and lo % 4 == 0
                 addr, off = a[1].split(" offset:")
                 tag = self.get(int(addr[1:]), "lds")
                 off = int(off)
-                assert tag[0] == "krd" and off % 4096 == 0 and off < 65536
-                slot, kb = off // g.K_TILE, (off % g.K_TILE) // 4096
+                assert tag[0] == "krd" and off % (16 * g.K_PITCH) == 0 and off < 65536
+                slot, kb = off // g.K_TILE, (off % g.K_TILE) // (16 * g.K_PITCH)
                 t = self.kslot[slot]
                 assert t is not None and ("K", slot) not in [(k, s) for k, s, _ in self.inflight], "K slot %d not readable (%s)" % (slot, ins)
                 self.seg_reads.add(("K", slot))
@@ -145,9 +152,9 @@ class Checker:
                 addr, off = a[1].split(" offset:")
                 tag = self.get(int(addr[1:]), "lds")
                 off = int(off)
-                assert tag[0] == "vrd" and off % 4096 == 0 and off < 65536
+                assert tag[0] == "vrd" and off % (16 * g.V_PITCH) == 0 and off < 65536
                 slot, rem = off // g.V_TILE, off % g.V_TILE
-                ps, half = rem // 8192, (rem % 8192) // 4096
+                ps, half = rem // (32 * g.V_PITCH), (rem % (32 * g.V_PITCH)) // (16 * g.V_PITCH)
                 t = self.vslot[slot]
                 assert t is not None and ("V", slot) not in [(k, s) for k, s, _ in self.inflight], "V slot %d not readable (%s)" % (slot, ins)
                 self.seg_reads.add(("V", slot))
@@ -172,7 +179,7 @@ class Checker:
                 ta, tb = self.get(int(a[1][1:]), "valu"), self.get(int(a[2][1:]), "valu")
                 assert ta[0] == "E" and tb[0] == "E" and ta[1:4] == tb[1:4] and ta[4] % 2 == 0 and tb[4] == ta[4] + 1, ins
                 t, kb, qb, j = ta[1], ta[2], ta[3], ta[4] // 2
-                assert d == g.p_reg(qb, kb // 2) + 2 * (kb % 2) + j, ins
+                assert d == g.p_reg(t, qb, kb // 2) + 2 * (kb % 2) + j, ins
                 self.put(d, ("Ph", t, qb, kb, j), self.p_need, "valu")
             elif op in ("v_dot2_f32_f16", "v_dot2c_f32_f16"):
                 d = int(a[0][1:])
@@ -260,7 +267,7 @@ class Checker:
                 addr, off = a[2].split(" offset:")
                 qt = self.get(int(a[1][1:]), "vmem")
                 assert addr == "%[qn]" and qt[0] == "qoff" and hi == lo + 3 and lo == g.q_reg(qt[1], int(off) // 64) and int(off) % 64 == 0, ins
-                assert self.n_qk == 32 * (self.n - 1), "Q overwritten before the last S = K.Q^T was issued"
+                assert self.n_qk == g.QKS * (self.n - 1), "Q overwritten before the last S = K.Q^T was issued"
                 for i in range(4): self.put(lo + i, ("Qnext", qt[1], int(off) // 64, i), 10 ** 9, "vmem")
                 self.vm_pending = True
             elif op == "s_addc_u32":
@@ -278,7 +285,7 @@ class Checker:
             assert ta == [("one",)] * 4 and a == g.ONES0, self.cur
             _, t, qb, kb0, _ = tb[0]
             ps = kb0 // 2
-            assert tb == [("Ph", t, qb, 2 * ps + j // 2, j % 2) for j in range(4)] and b == g.p_reg(qb, ps), self.cur
+            assert tb == [("Ph", t, qb, 2 * ps + j // 2, j % 2) for j in range(4)] and b == g.p_reg(t, qb, ps), self.cur
             assert d == g.LACC0 + 4 * qb and c == d, self.cur
             tc = [self.get(d + i, "mfma_c") for i in range(4)]
             n_prev = 0 if tc[0] == ("zero",) else tc[0][2]
@@ -303,23 +310,26 @@ class Checker:
             _, t, ps, db, _, _ = ta[0]
             assert ta == [("Vf", t, ps, db, h, i) for h in range(2) for i in range(2)], self.cur
             qb = tb[0][2]
-            assert tb == [("Ph", t, qb, 2 * ps + j // 2, j % 2) for j in range(4)] and b == g.p_reg(qb, ps), self.cur
-            assert d == g.o_reg(db, qb) and c == d, self.cur
+            assert tb == [("Ph", t, qb, 2 * ps + j // 2, j % 2) for j in range(4)] and b == g.p_reg(t, qb, ps), self.cur
+            assert d == self.o_id(db, qb) and c == d, self.cur
             tc = [self.get(d + i, "mfma_c") for i in range(4)]
             n_prev = 0 if tc[0] == ("zero",) else tc[0][3]
             assert all(x == ("zero",) for x in tc) or tc == [("O", db, qb, n_prev, i) for i in range(4)], self.cur
-            assert n_prev == 2 * t + ps, "O[%d][%d] accumulates tile %d half %d as its %d-th term" % (db, qb, t, ps, n_prev)
+            assert n_prev == g.PS * t + ps, "O[%d][%d] accumulates tile %d half %d as its %d-th term" % (db, qb, t, ps, n_prev)
             for i in range(4): self.put(d + i, ("O", db, qb, n_prev + 1, i), 1, "mfma")
+
+    def o_id(self, db, qb):
+        return (1000 if self.g.O_ACC else 0) + self.g.o_reg(db, qb)
 
     def finish(self):
         g, n = self.g, self.n
         for db in range(g.DB):
             for qb in range(g.QB):
-                for i in range(4): assert self.v[g.o_reg(db, qb) + i].tag == ("O", db, qb, 2 * n, i)
+                for i in range(4): assert self.v[self.o_id(db, qb) + i].tag == ("O", db, qb, g.PS * n, i)
         for qb in range(g.QB):
             if g.ROWSUM == "mfma": assert self.v[g.L_OUT[qb]].tag == ("lacc", qb, 2 * n, 0)
             else: assert self.v[g.L_OUT[qb]].tag == ("l", qb, n)
-        assert self.n_mfma == 32 * (n - 1) + (g.T - 32) * n
+        assert self.n_mfma == g.QKS * (n - 1) + (g.T - g.QKS) * n
         # the next work item: its first three K and two V tiles are on their way into slots 0-2 / 0-1, its Q is in the Q
         # registers, and everything has been waited for
         assert self.next_item == {"s40": True, "s42": True} and self.kptr == 3 and self.vptr == 2 and not self.kparts and not self.vparts
@@ -333,19 +343,22 @@ class Checker:
         assert self.idx - last_mfma > 8
 
 
-@pytest.mark.parametrize("rowsum", ["mfma", "add", "dot"])
+@pytest.mark.parametrize("shape,rowsum", [("d128", "mfma"), ("d128", "add"), ("d128", "dot"), ("d256", "add")])
 @pytest.mark.parametrize("n_tiles", [8, 12, 16, 32, 64])
-def test_loop_is_correct_symbolically(n_tiles, rowsum):
+def test_loop_is_correct_symbolically(n_tiles, shape, rowsum):
     g = _gen()
-    g.ROWSUM = rowsum
+    g.SHAPE, g.ROWSUM = shape, rowsum
     g.configure()
     c = Checker(g, n_tiles)
     c.run(g.program(n_tiles))
     c.finish()
 
 
-def test_checker_catches_a_broken_schedule():
+@pytest.mark.parametrize("shape", ["d128", "d256"])
+def test_checker_catches_a_broken_schedule(shape):
     g = _gen()
+    g.SHAPE = shape
+    g.configure()
     prog = g.program(8)
     # drop one LDS wait: some MFMA then reads a fragment that was not waited for
     k = next(i for i, ins in enumerate(prog) if ins.startswith("s_waitcnt lgkmcnt(") and i > 200)
@@ -357,7 +370,7 @@ def test_checker_catches_a_broken_schedule():
     # swap the operands of two neighbouring fragment reads
     k = next(i for i, ins in enumerate(prog) if ins.startswith("ds_read_b128") and i > 300)
     bad = list(prog)
-    bad[k] = re.sub(r"offset:(\d+)", lambda m: "offset:%d" % ((int(m.group(1)) + 4096) % 65536), bad[k])
+    bad[k] = re.sub(r"offset:(\d+)", lambda m: "offset:%d" % ((int(m.group(1)) + 16 * g.K_PITCH) % 65536), bad[k])
     with pytest.raises(AssertionError):
         c = Checker(g, 8)
         c.run(bad)
@@ -366,4 +379,4 @@ def test_checker_catches_a_broken_schedule():
 
 def test_committed_include_is_the_generators_output():
     r = subprocess.run([sys.executable, os.path.join(CSRC, "gen_fmha_loop16.py"), "--check"])
-    assert r.returncode == 0, "fmha_fwd_loop16_d128.inc is stale: run gen_fmha_loop16.py"
+    assert r.returncode == 0, "fmha_fwd_loop16_d128.inc / _d256.inc are stale: run gen_fmha_loop16.py"

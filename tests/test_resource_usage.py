@@ -29,7 +29,8 @@ AUTO_PICKED = {
     # fp16 head dim 64
     "fmha_fwd_kernel16<64,64,4,3,0,0,0,0,1,0,1,0>": (14, "the slow path of the row-sum test"),
     "fmha_fwd_kernel<64,64,4,3,0,0,0,0,1,0,0,0>": (0, ""),
-    # fp16 head dim 256
+    # fp16 head dim 256: big problems run the hand-scheduled persistent build (one wave per SIMD, O in accumulation registers)
+    "fmha_fwd_kernel16p<256,32,4,1,0,0,0,0,2,0,1,1>": (0, ""),
     "fmha_fwd_kernel<256,32,4,1,0,0,0,0,1,4,0,0>": (0, ""),
     "fmha_fwd_kernel<256,32,4,1,0,0,0,0,1,0,0,0>": (0, ""),
     # e4m3: big problems at head dim 128 from 4096 keys run the hand-scheduled persistent build (one register spilled once per

@@ -33,6 +33,10 @@ CASES = {
     # (half of the workgroups take a second item), 5x16x1024 = 320 with climbing keys (fall-back, then a next item)
     "256x128/16h": ["f16nt:1,512,2,128", "f16nt:1,256,3,128,768", "f16nt:2,2048,16,128", "f16nt:3,2048,16,128", "f16nt:1,512,2,128,1024",
                     "f16ntclimb:1,512,2,128,768", "f16ntclimb:5,1024,16,128", "f16:1,512,2,128", "f16:3,2048,16,128", "f16climb:1,512,2,128,768"],
+    # ... and its head-dim-256 shape (4 waves, one per SIMD, 32-key tiles; key length a multiple of 128, at least 256):
+    # 3x6 heads x 2048 rows = 288 items of 128 rows (32 workgroups take a second one), climbing keys, taps
+    "128x64/16h": ["f16nt:1,256,2,256", "f16nt:1,128,3,256,640", "f16nt:3,2048,6,256,512", "f16ntclimb:1,256,2,256,512",
+                   "f16ntclimb:3,1024,12,256,256", "f16:1,256,2,256,384", "f16climb:1,256,2,256,512"],
     # the e4m3 build with the hand-scheduled loop and persistent workgroups (key length a multiple of 256, from 4096): the
     # scheduled loop, 4352 keys (an odd number of loop turns), 2x10 heads x 4096 rows = 320 items (a quarter of the
     # workgroups take a second one), climbing keys (the vote, the max-tracking loop, then a next item: 5x13x1024 rows = 260)
@@ -97,7 +101,10 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     assert f.fmha_forward_kernel(f.CFK_FP16, 1, 8, 512, 512, 64) == "fmha_fwd_kernel_ks<64,8>"      # benchmark configuration 1
     assert f.fmha_forward_kernel(f.CFK_FP16, 2, 4, 512, 512, 128) == "fmha_fwd_kernel_ks<128,8>"
     assert f.fmha_forward_plan(f.CFK_FP16, 1, 2, 96, 192, 64)[:2] == (32, 64)                       # query rows a multiple of 32
-    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 8, 8192, 8192, 256) == 32
+    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 8, 8192, 8192, 256) == 16                             # hand-scheduled, 16x16x32
+    assert f.fmha_forward_kernel(f.CFK_FP16, 2, 8, 8192, 8192, 256) == "fmha_fwd_kernel16p<256,32,4,1,0,0,0,0,2,0,1,1>"
+    assert f.fmha_forward_kernel(f.CFK_FP16, 2, 8, 8192, 8160, 256) == "fmha_fwd_kernel<256,32,4,1,0,0,0,0,1,0,0,0>"   # key length % 128 != 0
+    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 256) == 32                              # medium problems: 32x32
     assert f.fmha_forward_mfma(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128) == 32
     assert f.fmha_forward_plan(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128)[:2] == (256, 128)
 
