@@ -130,7 +130,9 @@ def _make_fmha(pkg, w, seed=3080):
         kw.update(q_descale=qs, k_descale=ks, v_descale=vs)
     o = torch.empty((B, S, H, D), dtype=torch.float16, device=dev)
     flop = pkg.testbed.fmha_flops(B, H, S, S, D)
-    return (lambda: pkg.fmha_forward(q, k, v, o=o, **kw)), flop, (q, k, v, o, kw)
+    # the parameter block is filled in once; a step is then one cfk_fmha_forward call, as in the reference's launch loop
+    # (src/fmha-pipeline/fmha_forward.cu:578-592)
+    return pkg.fmha_forward(q, k, v, o=o, prepare=True, **kw), flop, (q, k, v, o, kw)
 
 
 def _make_gemm(pkg, w, seed=3080):

@@ -172,8 +172,9 @@ def _stream_ptr(stream):
 
 
 def fmha_forward(q, k, v, o=None, softmax_scale=None, q_descale=1.0, k_descale=1.0, v_descale=1.0,
-                 v_layout=CFK_V_BSHD, row_max=None, row_sum=None, scores=None, stream=None):
+                 v_layout=CFK_V_BSHD, row_max=None, row_sum=None, scores=None, stream=None, prepare=False):
     """O = softmax(scale * Q K^T) V on device tensors in [B,S,H,D] (D contiguous).
+    ``prepare=True`` launches nothing and returns a ``PreparedForward``: a callable that repeats this exact call.
 
     q,k,v: torch CUDA tensors, float16, or float8_e4m3fn / uint8 holding e4m3 codes (v may be float16 with e4m3
     q,k: hybrid mode).  ``v`` is [B,D,H,S] when
@@ -220,8 +221,30 @@ def fmha_forward(q, k, v, o=None, softmax_scale=None, q_descale=1.0, k_descale=1
                     dbg_row_max=row_max.data_ptr() if row_max is not None else 0,
                     dbg_row_sum=row_sum.data_ptr() if row_sum is not None else 0,
                     dbg_s=scores.data_ptr() if scores is not None else 0)
+    if prepare:
+        return PreparedForward(p, (q, k, v, o, row_max, row_sum, scores), stream)
     _check(lib().cfk_fmha_forward(ctypes.byref(p), _stream_ptr(stream)))
     return o
+
+
+class PreparedForward:
+    """One ``cfk_fmha_forward`` call with its parameter block filled in once (``fmha_forward(..., prepare=True)``): calling
+    the object launches it again on the stream given at preparation (torch's current stream then, if none was given).
+    What a C++ caller's launch loop does (src/fmha-pipeline/fmha_forward.cu:578-592): the checks and the ctypes
+    marshalling of ``fmha_forward`` cost several microseconds per call, as much as a small problem's kernel."""
+
+    def __init__(self, params, tensors, stream):
+        self.params, self.tensors = params, tensors   # (the tensors are held so that their memory stays alive)
+        self.o = tensors[3]
+        self._ref = ctypes.byref(params)
+        self._stream = _stream_ptr(stream)
+        self._fn = lib().cfk_fmha_forward
+
+    def __call__(self):
+        rc = self._fn(self._ref, self._stream)
+        if rc != 0:
+            _check(rc)
+        return self.o
 
 
 def gemm_f16(a, b, c=None, layout=CFK_GEMM_TN, stream=None):

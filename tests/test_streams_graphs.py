@@ -150,3 +150,19 @@ def test_init_makes_a_first_call_under_capture_possible():
         graph.replay()
         torch.cuda.synchronize()
         assert max_abs(o.float().cpu().numpy(), ref) <= TOL_FP16, rep
+
+
+@pytest.mark.gpu
+def test_prepared_call_repeats_the_same_launch():
+    # fmha_forward(..., prepare=True) fills the parameter block once; each call of the object is one cfk_fmha_forward
+    import torch
+    q, k, v = (to_dev(x.astype(np.float16)) for x in pkg.testbed.qkv(1, 256, 2, 64))
+    ref = pkg.fmha_forward(q, k, v)
+    o = torch.zeros_like(ref)
+    call = pkg.fmha_forward(q, k, v, o=o, prepare=True)
+    torch.cuda.synchronize()
+    assert float(o.abs().max()) == 0.0          # nothing was launched yet
+    for _ in range(3):
+        out = call()
+    torch.cuda.synchronize()
+    assert out is o and torch.equal(o, ref)
