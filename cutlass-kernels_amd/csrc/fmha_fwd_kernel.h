@@ -105,8 +105,9 @@ struct FmhaCfg {
   static_assert(SUB == 1 || SUB == 2, "sub-tiles per barrier");
   static_assert(!KPRE || SUB == 1, "K fragment prefetch is a variant of the one-tile step");
   static_assert(!ASM || ((M16 != (QK8 && PV8 && !VT)) && QK8 == PV8 && SUB == 2 &&
-                         ((D == 128 && BN == 64 && NWAVES == 8 && WPE == 2) || (M16 && D == 256 && BN == 32 && NWAVES == 4 && WPE == 1))),
-                "the hand-scheduled loops: fp16 on 16x16x32 MFMAs (head dims 128 and 256), e4m3 with V in [B,S,H,D] (128)");
+                         ((D == 128 && BN == 64 && NWAVES == 8 && WPE == 2) || (M16 && D == 256 && BN == 32 && NWAVES == 4 && WPE == 1) ||
+                          (M16 && D == 64 && BN == 64 && NWAVES == 8 && WPE == 2))),
+                "the hand-scheduled loops: fp16 on 16x16x32 MFMAs (head dims 64, 128, 256), e4m3 with V in [B,S,H,D] (128)");
   static_assert(BN % 32 == 0 && (!PV8 || BN == 64), "key tile: the e4m3 second GEMM has 64-deep K-steps");
   static_assert(!VT || PV8, "the pre-transposed layout is an e4m3-V layout");
   static_assert(K_IPW >= 1 && K_IPW * K_RPI * NWAVES == BN && V_IPW >= 1 && V_IPW * V_RPI * NWAVES == V_ROWS,

@@ -1,12 +1,15 @@
 #!/usr/bin/env python3
 """Generator of the hand-scheduled main loops of the fp16 FMHA forward kernel on 16x16x32 MFMAs (fmha_fwd_kernel16p.h,
-FmhaCfg::ASM), in two shapes:
+FmhaCfg::ASM), in three shapes:
   d128  head dim 128, 64-key tiles, 256 query rows per workgroup (8 waves x 32 rows, two waves per SIMD)
+  d64   head dim 64, 64-key tiles of 8 KB, 256 query rows per workgroup (8 waves, two per SIMD); 36 MFMA slots per tile:
+        here the softmax (112 vector instructions beside 32 MFMAs) is what fills the issue port, so the row sum goes to
+        the matrix pipe (ROWSUM = "mfma")
   d256  head dim 256, 32-key tiles, 128 query rows per workgroup (4 waves x 32 rows, one wave per SIMD: Q and O alone
         are 192 registers per lane; O lives in the accumulation registers a[0:127])
-Both have the same timeline (64 MFMA slots and 16 KB of K and of V per tile); the text below describes d128.
+d128 and d256 have the same timeline (64 MFMA slots and 16 KB of K and of V per tile); the text below describes d128.
 
-    python3 gen_fmha_loop16.py            # rewrites fmha_fwd_loop16_d128.inc and fmha_fwd_loop16_d256.inc beside this file
+    python3 gen_fmha_loop16.py            # rewrites fmha_fwd_loop16_{d128,d256,d64}.inc beside this file
     python3 gen_fmha_loop16.py --check    # exit status 1 if those files are not what the generator produces
 
 Why a generator: the loop is one inline-asm statement of ~2800 instructions with every register assigned by hand.
@@ -63,8 +66,7 @@ import sys
 # ---- shape --------------------------------------------------------------------------------------------------------
 SHAPE = "d128"
 QB, NSLOT = 2, 4
-K_TILE = V_TILE = 16384                 # both shapes: 64 keys x 256 B = 32 keys x 512 B
-K_ST0, V_ST0 = 0, NSLOT * K_TILE        # LDS map: K slots, then V slots (the read addresses include these bases)
+K_ST0 = 0                               # LDS map: K slots, then V slots (the read addresses include these bases)
 
 # ---- how the row sum l is taken ----------------------------------------------------------------------------------
 #   "mfma": l += 1 . P on the matrix pipe (sums P as rounded to fp16, the weights the second GEMM applies)
@@ -85,15 +87,22 @@ def configure():
     g = globals()
     if SHAPE == "d128":
         g.update(D=128, BN=64, NWAVES=8, O_ACC=False, O0=192, SA0=128, SB0=160, Q0=96, P0=80, RING0=48, KRD0=24, VRD0=28, GOK0=36, GOV0=38)
+    elif SHAPE == "d64":
+        assert ROWSUM == "mfma"
+        g.update(D=64, BN=64, NWAVES=8, O_ACC=False, O0=224, SA0=160, SB0=192, Q0=144, P0=128, RING0=96, KRD0=82, VRD0=78, GOK0=77, GOV0=76)
     else:
         assert ROWSUM == "add"
         g.update(D=256, BN=32, NWAVES=4, O_ACC=True, O0=0, SA0=224, SB0=240, Q0=160, P0=144, RING0=112, KRD0=96, VRD0=80, GOK0=72, GOV0=76)
     g.update(KB=BN // 16, KS=D // 32, DB=D // 16, PS=BN // 32, K_PITCH=2 * D, V_PITCH=2 * D)
+    g.update(K_TILE=BN * K_PITCH, V_TILE=BN * V_PITCH, V_ST0=NSLOT * BN * K_PITCH)
     g["IPW"] = K_TILE // 1024 // NWAVES     # copies per wave and tile (K and V alike)
     g["QKS"] = KS * KB * QB                 # MFMA slots of S = K.Q^T
     if SHAPE == "d256":
         g.update(M0R=70, LA0=64, QOFF0=68, LOW=64, L_OUT=(64, 66), T=64, L_TOTAL=False)
         start = 36   # S(t+1) is complete at slot 32; P(t+1) has to be before slot 32 of the next period
+    elif SHAPE == "d64":
+        g.update(M0R=74, ONES0=92, LACC0=84, QOFF0=72, LOW=72, L_OUT=(84, 88), T=36, L_TOTAL=True)
+        start = 23   # P(t)'s first half is consumed by slot 26; P(t+1)'s second half is needed at slot 26 of the next period
     elif ROWSUM == "mfma":
         g.update(M0R=18, ONES0=20, LACC0=40, QOFF0=16, LOW=16, L_OUT=(40, 44), T=68, L_TOTAL=True)
         start = 46
@@ -386,8 +395,8 @@ configure()
 if __name__ == "__main__":
     overrides = json.loads(os.environ.get("LOOP16_SET", "{}"))
     stale = False
-    for shape in ("d128", "d256"):
-        SHAPE = shape
+    for shape, rowsum in (("d128", "add"), ("d256", "add"), ("d64", "mfma")):
+        SHAPE, ROWSUM = shape, rowsum
         for k, v in overrides.items(): globals()[k] = v
         configure()
         out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fmha_fwd_loop16_%s.inc" % shape)

@@ -1,5 +1,6 @@
 """Symbolic check of the hand-scheduled main loops of the fp16 kernel (cutlass-kernels_amd/csrc/gen_fmha_loop16.py), in
-both of its shapes (head dim 128: 8 waves, 64-key tiles; head dim 256: 4 waves, 32-key tiles, O in accumulation registers).
+its three shapes (head dim 128: 8 waves, 64-key tiles; head dim 256: 4 waves, 32-key tiles, O in accumulation registers;
+head dim 64: 8 waves, 64-key tiles of 8 KB, row sum on the matrix pipe).
 
 A loop is ~2800 hand-allocated instructions inside one asm statement, where neither the compiler's register
 allocator nor its hazard recognizer helps.  This test walks the instruction text a wave executes (loop unrolled for
@@ -343,7 +344,7 @@ class Checker:
         assert self.idx - last_mfma > 8
 
 
-@pytest.mark.parametrize("shape,rowsum", [("d128", "mfma"), ("d128", "add"), ("d128", "dot"), ("d256", "add")])
+@pytest.mark.parametrize("shape,rowsum", [("d128", "mfma"), ("d128", "add"), ("d128", "dot"), ("d256", "add"), ("d64", "mfma")])
 @pytest.mark.parametrize("n_tiles", [8, 12, 16, 32, 64])
 def test_loop_is_correct_symbolically(n_tiles, shape, rowsum):
     g = _gen()
@@ -354,10 +355,10 @@ def test_loop_is_correct_symbolically(n_tiles, shape, rowsum):
     c.finish()
 
 
-@pytest.mark.parametrize("shape", ["d128", "d256"])
+@pytest.mark.parametrize("shape", ["d128", "d256", "d64"])
 def test_checker_catches_a_broken_schedule(shape):
     g = _gen()
-    g.SHAPE = shape
+    g.SHAPE, g.ROWSUM = shape, ("mfma" if shape == "d64" else "add")
     g.configure()
     prog = g.program(8)
     # drop one LDS wait: some MFMA then reads a fragment that was not waited for
@@ -379,4 +380,4 @@ def test_checker_catches_a_broken_schedule(shape):
 
 def test_committed_include_is_the_generators_output():
     r = subprocess.run([sys.executable, os.path.join(CSRC, "gen_fmha_loop16.py"), "--check"])
-    assert r.returncode == 0, "fmha_fwd_loop16_d128.inc / _d256.inc are stale: run gen_fmha_loop16.py"
+    assert r.returncode == 0, "fmha_fwd_loop16_{d128,d256,d64}.inc are stale: run gen_fmha_loop16.py"

@@ -32,7 +32,10 @@ CASES = {
     # max-tracking loop that serves the taps; 2x16 heads x 2048 rows = 256 items (one per workgroup), 3x16x2048 = 384
     # (half of the workgroups take a second item), 5x16x1024 = 320 with climbing keys (fall-back, then a next item)
     "256x128/16h": ["f16nt:1,512,2,128", "f16nt:1,256,3,128,768", "f16nt:2,2048,16,128", "f16nt:3,2048,16,128", "f16nt:1,512,2,128,1024",
-                    "f16ntclimb:1,512,2,128,768", "f16ntclimb:5,1024,16,128", "f16:1,512,2,128", "f16:3,2048,16,128", "f16climb:1,512,2,128,768"],
+                    "f16ntclimb:1,512,2,128,768", "f16ntclimb:5,1024,16,128", "f16:1,512,2,128", "f16:3,2048,16,128", "f16climb:1,512,2,128,768",
+                    # ... its head-dim-64 shape (row sum on the matrix pipe)
+                    "f16nt:1,512,2,64", "f16nt:1,256,3,64,768", "f16nt:3,2048,16,64", "f16ntclimb:1,512,2,64,768", "f16ntclimb:5,1024,16,64",
+                    "f16:1,512,2,64", "f16climb:1,512,2,64,1024"],
     # ... and its head-dim-256 shape (4 waves, one per SIMD, 32-key tiles; key length a multiple of 128, at least 256):
     # 3x6 heads x 2048 rows = 288 items of 128 rows (32 workgroups take a second one), climbing keys, taps
     "128x64/16h": ["f16nt:1,256,2,256", "f16nt:1,128,3,256,640", "f16nt:3,2048,6,256,512", "f16ntclimb:1,256,2,256,512",
@@ -82,7 +85,7 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     assert shapes("128x64") == "32 32 32 32 (128, 64)"
     assert shapes("256x128") == "32 32 32 32 (256, 128)"
     assert shapes("256x128/16") == "16 32 32 32 (256, 128)"   # two key tiles per barrier on 16x16x32: head dim 128 only
-    assert shapes("256x128/16h") == "16 32 32 32 (256, 128)"  # ... with the hand-scheduled loop
+    assert shapes("256x128/16h") == "16 16 32 32 (256, 128)"  # ... with the hand-scheduled loop: head dims 128 and 64
     # the hand-scheduled build needs 160 KB of LDS; a wish for the compiler-scheduled one (no `h`) is kept apart from it
     lds_code = ("import sys; sys.path.insert(0, %r); import __graft_entry__ as e; p = e.load_package(); f = p.fmha; "
                 "print(f.fmha_forward_plan(f.CFK_FP16, 2, 4, 1536, 512, 128)[2], f.fmha_forward_plan(f.CFK_FP16, 2, 4, 1536, 384, 128)[:3])" % ROOT)
@@ -96,7 +99,9 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     # ... on 16x16x32 MFMAs for fp16 at head dims 64 and 128; small problems, head dim 256 and e4m3 stay on 32x32
     assert f.fmha_forward_mfma(f.CFK_FP16, 8, 16, 2048, 2048, 128) == 16
     assert f.fmha_forward_mfma(f.CFK_FP16, 4, 32, 4096, 4096, 64) == 16
-    assert f.fmha_forward_plan(f.CFK_FP16, 4, 32, 4096, 4096, 64)[:2] == (128, 64)
+    assert f.fmha_forward_plan(f.CFK_FP16, 4, 32, 4096, 4096, 64)[:2] == (256, 128)      # hand-scheduled
+    assert f.fmha_forward_kernel(f.CFK_FP16, 4, 32, 4096, 4096, 64) == "fmha_fwd_kernel16p<64,64,8,2,0,0,0,0,2,0,1,1>"
+    assert f.fmha_forward_plan(f.CFK_FP16, 4, 32, 4096, 4032, 64)[:2] == (128, 64)       # key length % 256 != 0
     assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 128) == 32
     assert f.fmha_forward_kernel(f.CFK_FP16, 1, 8, 512, 512, 64) == "fmha_fwd_kernel_ks<64,8>"      # benchmark configuration 1
     assert f.fmha_forward_kernel(f.CFK_FP16, 2, 4, 512, 512, 128) == "fmha_fwd_kernel_ks<128,8>"
