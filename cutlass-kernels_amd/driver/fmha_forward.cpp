@@ -273,7 +273,10 @@ int main(int argc, char **argv) {
   }
   int mfma = 0;
   cfk_fmha_forward_mfma(&plan_q, &mfma);
-  printf("M = %d\nN = %d\nK = %d\nQBLK = %d\nKBLK = %d\nMFMA = %dx%d\nL = %d : %d * %d\n", S, S, D, bm, bn, mfma, mfma, H * B, H, B);
+  char kernel_name[96] = "";
+  cfk_fmha_forward_kernel(&plan_q, kernel_name, (int32_t)sizeof kernel_name);
+  printf("M = %d\nN = %d\nK = %d\nQBLK = %d\nKBLK = %d\nMFMA = %dx%d\nKERNEL = %s\nL = %d : %d * %d\n", S, S, D, bm, bn, mfma, mfma, kernel_name,
+         H * B, H, B);
 
   // seeded N(0,1) inputs, seeds 3080 + {1,2,3} (fmha_forward.cu:479-500)
   const size_t n = (size_t)B * S * H * D;

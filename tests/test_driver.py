@@ -102,20 +102,23 @@ def test_sweep_script_verify_all_on_a_reduced_problem():
     r = subprocess.run(["bash", script, "verify-all"], env=env, capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout[-4000:] + r.stderr[-2000:]
     blocks = r.stdout.split("CONFIG ")[1:]
-    assert len(blocks) == 32, len(blocks)
+    assert len(blocks) == 38, len(blocks)
     seen = set()
     for blk in blocks:
         head_line = blk.splitlines()[0]
         mode, head, tile = (x.split("=")[1] for x in head_line.replace(",", "").split())
-        shape, _, mfma = tile.partition("/")          # <query rows>x<keys>[/16]: the build on 16x16x32 MFMAs
+        shape, _, mfma = tile.partition("/")          # <query rows>x<keys>[/16|/16h|/32h]: MFMA shape, hand-scheduled loop
         bm, bn = shape.split("x")
+        hand = mfma.endswith("h")
+        mfma = mfma.rstrip("h") or ("16" if bm == "32" else "32")            # (the 32-row build runs on 16x16x32 MFMAs)
         assert f"QBLK = {bm}" in blk and f"KBLK = {bn}" in blk, blk          # the wished tile is the one that ran
-        assert f"MFMA = {mfma or 32}x{mfma or 32}" in blk, blk
+        assert f"MFMA = {mfma}x{mfma}" in blk, blk
+        assert ("kernel16p<" in blk or "kernel8p<" in blk) == hand, blk      # ... and the wished kind of kernel
         for line in ("gemm-check-1: Passed", "max-check: Passed", "sum-check: Passed", "gemm-check-2: Passed"):
             assert line in blk, (head_line, blk)
         assert "Failed" not in blk
         seen.add((mode, head, tile))
-    assert len(seen) == 32
+    assert len(seen) == 38
     assert {m for m, _, _ in seen} == {"fp16", "fp8", "fp8-bdhs", "hybrid"}
 
 
