@@ -9,5 +9,5 @@ The directory name is not a Python identifier; load it with ``__graft_entry__.lo
 repository root on ``sys.path`` and use ``importlib`` as that helper does.
 """
 from . import fmha, testbed  # noqa: F401
-from .fmha import (CFK_FP16, CFK_FP32, CFK_FP8_E4M3, CfkError, build, fmha_forward, fmha_forward_mfma, fmha_forward_plan,  # noqa: F401
-                   gemm, gemm_f16, last_error, lib, lib_path, version)
+from .fmha import (CFK_FP16, CFK_FP32, CFK_FP8_E4M3, CfkError, build, fmha_forward, fmha_forward_kernel, fmha_forward_mfma,  # noqa: F401
+                   fmha_forward_plan, gemm, gemm_f16, last_error, lib, lib_path, version)

@@ -151,10 +151,10 @@ def test_invariants_on_device():
     assert max_abs(o.float().cpu().numpy(), base) == 0.0
 
 
-def _subset_check(B, S, H, D, climb=False):
+def _subset_check(B, S, H, D, climb=False, **climb_kw):
     q, k, v = pkg.testbed.qkv(B, S, H, D)
     if climb:
-        k, v = climbing_keys(k), v / 4
+        k, v = climbing_keys(k, **climb_kw), v / 4
     got, (qf, kf, vf) = _run(q, k, v)
     pairs = subset_pairs(B, H)
     ref = oracle.attention_f32(qf, kf, vf, bh_pairs=pairs)["O"]
@@ -179,6 +179,16 @@ def test_headline_shapes_with_climbing_scores():
     # reference point
     _subset_check(8, 2048, 16, 128, climb=True)
     _subset_check(4, 2048, 16, 64, climb=True)
+
+
+@pytest.mark.parametrize("B,S,H,D,ramp", [(8, 1024, 16, 128, 8.0), (8, 1024, 16, 128, 4.5), (4, 2048, 16, 64, 8.0),
+                                          (2, 8192, 8, 256, 8.0)])
+def test_weights_beyond_fp16_but_within_fp32(B, S, H, D, ramp):
+    # No spike key: the scores climb 15 to 35 binades above the first tile's row max, so the weights taken against that
+    # fixed reference point overflow fp16 (P) but not fp32 -- a sum of the fp32 weights stays finite, and the test that
+    # sends a workgroup to the max-tracking loop has to go by its size.  Ramp 4.5: only some rows get that far.
+    assert "kernel16p<" in pkg.fmha_forward_kernel(pkg.CFK_FP16, B, H, S, S, D)     # the fixed reference point is theirs
+    _subset_check(B, S, H, D, climb=True, ramp=ramp, spike=1.0)
 
 
 def test_config3_long_sequence_large_head_subset_check():
