@@ -73,6 +73,10 @@ K_ST0 = 0                               # LDS map: K slots, then V slots (the re
 #   "add":  v_add_f32 over the fp32 weights before the cast (online_softmax.h:173-206), two chains per query block
 #   "dot":  v_dot2c_f32_f16 over the rounded weights, summed per tile in the order of fmha_fwd_kernel16.h's loop
 ROWSUM = "add"
+# FOLD: Q arrives multiplied by the softmax scale c and S = K.Q^T starts from -m (the C operand of the first K-step is
+# a register quad that holds -m) instead of from zero: the scores leave the matrix pipe as c S - m and the softmax has
+# no multiply-add per score.  The caller subtracts m from S(0) itself.  (Only for the row-sum forms of the product.)
+FOLD = True
 RING = 8
 LOOKAHEAD = 7      # fragments requested ahead of use
 HOLD = 4           # MFMAs of a super-step issued behind its barrier
@@ -97,15 +101,19 @@ def configure():
     g.update(K_TILE=BN * K_PITCH, V_TILE=BN * V_PITCH, V_ST0=NSLOT * BN * K_PITCH)
     g["IPW"] = K_TILE // 1024 // NWAVES     # copies per wave and tile (K and V alike)
     g["QKS"] = KS * KB * QB                 # MFMA slots of S = K.Q^T
+    g["FOLDED"] = FOLD and (SHAPE, ROWSUM) in (("d128", "add"), ("d256", "add"), ("d64", "mfma"))
     if SHAPE == "d256":
-        g.update(M0R=70, LA0=64, QOFF0=68, LOW=64, L_OUT=(64, 66), T=64, L_TOTAL=False)
+        g.update(M0R=70, MN0=104, LA0=64, QOFF0=68, LOW=64, L_OUT=(64, 66), T=64, L_TOTAL=False)
         start = 36   # S(t+1) is complete at slot 32; P(t+1) has to be before slot 32 of the next period
     elif SHAPE == "d64":
-        g.update(M0R=74, ONES0=92, LACC0=84, QOFF0=72, LOW=72, L_OUT=(84, 88), T=36, L_TOTAL=True)
+        g.update(M0R=74, MN0=64, ONES0=92, LACC0=84, QOFF0=72, LOW=64 if FOLDED else 72, L_OUT=(84, 88), T=36, L_TOTAL=True)
         start = 23   # P(t)'s first half is consumed by slot 26; P(t+1)'s second half is needed at slot 26 of the next period
     elif ROWSUM == "mfma":
         g.update(M0R=18, ONES0=20, LACC0=40, QOFF0=16, LOW=16, L_OUT=(40, 44), T=68, L_TOTAL=True)
         start = 46
+    elif ROWSUM == "add" and FOLDED:
+        g.update(MN0=40, LA0=18, QOFF0=22, LOW=18, L_OUT=(18, 20), T=64, L_TOTAL=False)
+        start = 44
     elif ROWSUM == "add":
         g.update(M0R=40, LA0=42, QOFF0=22, LOW=22, L_OUT=(42, 44), T=64, L_TOTAL=False)
         start = 44
@@ -145,7 +153,8 @@ class Frag:
     def mfma(self, qb):
         if self.kind == 'K':
             d = s_reg(self.t, self.b, qb)
-            return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (vr(d), vr(self.reg), vr(q_reg(qb, self.a)), "0" if self.a == 0 else vr(d))
+            c0 = vr(MN0 + 4 * qb) if FOLDED else "0"
+            return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (vr(d), vr(self.reg), vr(q_reg(qb, self.a)), c0 if self.a == 0 else vr(d))
         d = o_txt(self.b, qb)
         return "v_mfma_f32_16x16x32_f16 %s, %s, %s, %s" % (d, vr(self.reg), vr(p_reg(self.t, qb, self.a)), d)
 
@@ -162,7 +171,8 @@ def softmax_ops(t):
         for qb in range(QB):
             s = s_reg(t, kb, qb)
             p = p_reg(t, qb, kb // 2) + 2 * (kb % 2)
-            for i in range(4): ops.append(("v_fma_f32 v%d, v%d, %%[c], -v%d" % (s + i, s + i, M0R + qb), 1))
+            if not FOLDED:
+                for i in range(4): ops.append(("v_fma_f32 v%d, v%d, %%[c], -v%d" % (s + i, s + i, M0R + qb), 1))
             for i in range(4): ops.append(("v_exp_f32 v%d, v%d" % (s + i, s + i), 2))
             if ROWSUM == "add" and "rowsum" not in ABLATE:
                 for i in range(4): ops.append(("v_add_f32 v%d, v%d, v%d" % (LA0 + 2 * qb + i % 2, LA0 + 2 * qb + i % 2, s + i), 1))
@@ -289,6 +299,9 @@ def schedule(n_tiles):
         for r in range(LA0, LA0 + 4): cur.append("v_mov_b32 v%d, 0" % r)
     else:
         for qb in range(QB): cur.append("v_mov_b32 v%d, 0" % (L0 + qb))
+    if FOLDED:   # -m of a query block, in the four registers of an MFMA's C operand (the caller fills the first)
+        for qb in range(QB):
+            for i in range(1, 4): cur.append("v_mov_b32 v%d, v%d" % (MN0 + 4 * qb + i, MN0 + 4 * qb))
     if "reads" in ABLATE:
         for r in range(RING0, RING0 + 4 * RING): cur.append("v_mov_b32 v%d, 0" % r)
     request(0, LOOKAHEAD)
@@ -350,13 +363,17 @@ def render():
     in scope: bool sum_is_complete (out: the flag), f32x16 o0, o1, .. (out: the O accumulators, 16 registers each, in register order), sa0, .. (in, clobbered:
     S(0)), q0, .. (in: this item's Q; out: the next item's); float l0, l1 (out); uint64_t kptr, vptr (in: this item's K
     tile 3 / V tile 2; out: the same of the next item), kn, vn, qn (the next item's K, V and this wave's Q rows);
-    uint32_t nloop, k_rd[KS], v_rd[DB], goff_k[IPW], goff_v[IPW], qoff[2], lds_wave, tile_stride; float m_ref[2], c_log2."""
+    uint32_t nloop, k_rd[KS], v_rd[DB], goff_k[IPW], goff_v[IPW], qoff[2], lds_wave, tile_stride; float m_ref[2], c_log2
+    (FOLD: float m_neg[2] instead of those two); constexpr bool kFold."""
     head, body, tail = folded()
     L = []
     L.append("// GENERATED by gen_fmha_loop16.py -- do not edit.  The hand-scheduled main loop of fmha_fwd_kernel16p (FmhaCfg::ASM: head")
     L.append("// dim %d, %d x %d): %d + %d (loop) + %d instructions, row sum by \"%s\"." % (D, 32 * NWAVES, 2 * BN, len(head), len(body), len(tail), ROWSUM))
     L.append("// l0 / l1 hold the complete row sum of the lane's query in every lane (true) or the lane's share of it (false)")
     L.append("sum_is_complete = %s;" % ("true" if L_TOTAL else "false"))
+    L.append("// Q is expected multiplied by the softmax scale, S(0) with the reference point taken off, m_neg[] = minus that point (true);")
+    L.append("// or Q and S(0) as they are, m_ref[] = the reference point (false)")
+    L.append("static_assert(kFold == %s, \"the caller prepares Q, S(0) and the reference point in the form this loop takes\");" % ("true" if FOLDED else "false"))
     L.append("asm volatile(")
     def emit(ins): L.append('    "%s\\n"' % ins)
     for i in head: emit(i)
@@ -379,12 +396,17 @@ def render():
     ins = ['"{v%d}"(qoff[%d])' % (QOFF0 + i, i) for i in range(QB)] + ['[kn] "s"(kn)', '[vn] "s"(vn)', '[qn] "s"(qn)']
     ins += ['"{v%d}"(k_rd[%d])' % (KRD0 + i, i) for i in range(KS)] + ['"{v%d}"(v_rd[%d])' % (VRD0 + i, i) for i in range(DB)]
     ins += ['"{v%d}"(goff_k[%d])' % (GOK0 + i, i) for i in range(IPW)] + ['"{v%d}"(goff_v[%d])' % (GOV0 + i, i) for i in range(IPW)]
-    ins += ['"{v%d}"(m_ref[%d])' % (M0R + i, i) for i in range(QB)]
-    ins += ['[c] "s"(c_log2)', '[ldsw] "s"(lds_wave)', '[stride] "s"(tile_stride)']
+    if FOLDED:
+        ins += ['"{v%d}"(m_neg[%d])' % (MN0 + 4 * i, i) for i in range(QB)]
+        ins += ['[ldsw] "s"(lds_wave)', '[stride] "s"(tile_stride)']
+    else:
+        ins += ['"{v%d}"(m_ref[%d])' % (M0R + i, i) for i in range(QB)]
+        ins += ['[c] "s"(c_log2)', '[ldsw] "s"(lds_wave)', '[stride] "s"(tile_stride)']
     if ROWSUM == "dot": ins.append('[ones] "s"(0x3c003c00u)')
     L.append("    : " + ", ".join(ins))
     used = set(range(SA0, SA0 + 16 * n_s)) | set(range(Q0, Q0 + 16 * n_q)) | set(range(KRD0, KRD0 + KS)) | set(range(VRD0, VRD0 + DB))
-    used |= set(range(GOK0, GOK0 + IPW)) | set(range(GOV0, GOV0 + IPW)) | {M0R, M0R + 1, QOFF0, QOFF0 + 1} | set(L_OUT)
+    used |= set(range(GOK0, GOK0 + IPW)) | set(range(GOV0, GOV0 + IPW)) | {QOFF0, QOFF0 + 1} | set(L_OUT)
+    used |= {MN0, MN0 + 4} if FOLDED else {M0R, M0R + 1}
     if not O_ACC: used |= set(range(O0, O0 + 16 * n_o))
     clob = ['"memory"', '"scc"', '"m0"'] + ['"v%d"' % r for r in range(LOW, 256) if r not in used]
     L.append("    : " + ", ".join(clob) + ");")

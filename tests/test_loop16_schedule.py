@@ -63,7 +63,8 @@ class Checker:
         for qb in range(g.QB):
             for s in range(g.KS):
                 for i in range(4): self.put(g.q_reg(qb, s) + i, ("Q", qb, s, i), 10 ** 9, "init")
-            self.put(g.M0R + qb, ("m", qb), 10 ** 9, "init")
+            if g.FOLDED: self.put(g.MN0 + 4 * qb, ("mneg", qb), 10 ** 9, "init")
+            else: self.put(g.M0R + qb, ("m", qb), 10 ** 9, "init")
             self.put(g.QOFF0 + qb, ("qoff", qb), 10 ** 9, "init")
         self.e_need = 2 if g.ROWSUM == "add" else 1                 # uses of an exponential: the convert (+ the add)
         self.p_need = g.DB + (0 if g.ROWSUM == "add" else 1)        # uses of a packed weight: 8 MFMAs (+ the row sum)
@@ -128,6 +129,10 @@ class Checker:
                     assert (kind, slot) not in self.seg_reads, "%s slot %d copied and read in one barrier interval" % (kind, slot)
                     (self.kslot if kind == "K" else self.vslot)[slot] = t
                 self.inflight, self.seg_reads = [], set()
+            elif op == "v_mov_b32" and a[1].startswith("v"):
+                tag = self.get(int(a[1][1:]), "valu")
+                assert g.FOLDED and tag[0] == "mneg" and 0 < int(a[0][1:]) - (g.MN0 + 4 * tag[1]) < 4, ins
+                self.put(int(a[0][1:]), tag, 10 ** 9, "valu")
             elif op == "v_mov_b32":
                 assert a[1] in ("0", "0x3c003c00")
                 self.put(int(a[0][1:]), ("zero",) if a[1] == "0" else ("one",), 10 ** 9, "valu")
@@ -165,7 +170,7 @@ class Checker:
                 self.mfma(R(a[0])[0], R(a[1])[0], R(a[2])[0], None if a[3] == "0" else R(a[3])[0])
             elif op == "v_fma_f32":
                 d, s_ = int(a[0][1:]), int(a[1][1:])
-                assert d == s_ and a[2] == "%[c]" and a[3].startswith("-v")
+                assert not g.FOLDED and d == s_ and a[2] == "%[c]" and a[3].startswith("-v")
                 tag = self.get(s_, "valu")
                 mt = self.get(int(a[3][2:]), "valu")
                 assert tag[0] == "S" and tag[4] == g.KS - 1 and d == g.s_reg(tag[1], tag[2], tag[3]) + tag[5] and mt == ("m", tag[3]), ins
@@ -173,6 +178,9 @@ class Checker:
             elif op == "v_exp_f32":
                 d, s_ = int(a[0][1:]), int(a[1][1:])
                 tag = self.get(s_, "valu")
+                if g.FOLDED:   # the score comes off the matrix pipe scaled and with the reference point taken off
+                    assert tag[0] == "S" and tag[4] == g.KS - 1 and d == g.s_reg(tag[1], tag[2], tag[3]) + tag[5], ins
+                    tag = ("X",) + tag[1:4] + (tag[5],)
                 assert d == s_ and tag[0] == "X", ins
                 self.put(d, ("E",) + tag[1:], self.e_need, "trans")
             elif op == "v_cvt_pk_f16_f32":
@@ -300,7 +308,9 @@ class Checker:
             assert tb == [("Q", qb, s, i) for i in range(4)] and b == g.q_reg(qb, s), self.cur
             assert d == g.s_reg(t, kb, qb), self.cur
             self.n_qk += 1
-            if s == 0:
+            if s == 0 and g.FOLDED:
+                assert c == g.MN0 + 4 * qb and [self.get(c + i, "mfma_c") for i in range(4)] == [("mneg", qb)] * 4, self.cur
+            elif s == 0:
                 assert c is None, self.cur
             else:
                 assert c == d
@@ -344,12 +354,14 @@ class Checker:
         assert self.idx - last_mfma > 8
 
 
-@pytest.mark.parametrize("shape,rowsum", [("d128", "mfma"), ("d128", "add"), ("d128", "dot"), ("d256", "add"), ("d64", "mfma")])
+@pytest.mark.parametrize("shape,rowsum,fold", [("d128", "mfma", False), ("d128", "add", True), ("d128", "add", False), ("d128", "dot", False),
+                                               ("d256", "add", True), ("d256", "add", False), ("d64", "mfma", True), ("d64", "mfma", False)])
 @pytest.mark.parametrize("n_tiles", [8, 12, 16, 32, 64])
-def test_loop_is_correct_symbolically(n_tiles, shape, rowsum):
+def test_loop_is_correct_symbolically(n_tiles, shape, rowsum, fold):
     g = _gen()
-    g.SHAPE, g.ROWSUM = shape, rowsum
+    g.SHAPE, g.ROWSUM, g.FOLD = shape, rowsum, fold
     g.configure()
+    assert g.FOLDED == fold
     c = Checker(g, n_tiles)
     c.run(g.program(n_tiles))
     c.finish()
