@@ -75,7 +75,7 @@ K_ST0 = 0                               # LDS map: K slots, then V slots (the re
 ROWSUM = "add"
 # FOLD: Q arrives multiplied by the softmax scale c and S = K.Q^T starts from -m (the C operand of the first K-step is
 # a register quad that holds -m) instead of from zero: the scores leave the matrix pipe as c S - m and the softmax has
-# no multiply-add per score.  The caller subtracts m from S(0) itself.  (Only for the row-sum forms of the product.)
+# no multiply-add per score.  The caller subtracts m from S(0) itself.  (Not with ROWSUM = "dot".)
 FOLD = True
 RING = 8
 LOOKAHEAD = 7      # fragments requested ahead of use
@@ -101,13 +101,16 @@ def configure():
     g.update(K_TILE=BN * K_PITCH, V_TILE=BN * V_PITCH, V_ST0=NSLOT * BN * K_PITCH)
     g["IPW"] = K_TILE // 1024 // NWAVES     # copies per wave and tile (K and V alike)
     g["QKS"] = KS * KB * QB                 # MFMA slots of S = K.Q^T
-    g["FOLDED"] = FOLD and (SHAPE, ROWSUM) in (("d128", "add"), ("d256", "add"), ("d64", "mfma"))
+    g["FOLDED"] = FOLD and ROWSUM != "dot"
     if SHAPE == "d256":
         g.update(M0R=70, MN0=104, LA0=64, QOFF0=68, LOW=64, L_OUT=(64, 66), T=64, L_TOTAL=False)
         start = 36   # S(t+1) is complete at slot 32; P(t+1) has to be before slot 32 of the next period
     elif SHAPE == "d64":
         g.update(M0R=74, MN0=64, ONES0=92, LACC0=84, QOFF0=72, LOW=64 if FOLDED else 72, L_OUT=(84, 88), T=36, L_TOTAL=True)
         start = 23   # P(t)'s first half is consumed by slot 26; P(t+1)'s second half is needed at slot 26 of the next period
+    elif ROWSUM == "mfma" and FOLDED:
+        g.update(MN0=12, ONES0=20, LACC0=40, QOFF0=10, LOW=10, L_OUT=(40, 44), T=68, L_TOTAL=True)
+        start = 46
     elif ROWSUM == "mfma":
         g.update(M0R=18, ONES0=20, LACC0=40, QOFF0=16, LOW=16, L_OUT=(40, 44), T=68, L_TOTAL=True)
         start = 46
@@ -417,9 +420,12 @@ configure()
 if __name__ == "__main__":
     overrides = json.loads(os.environ.get("LOOP16_SET", "{}"))
     stale = False
+    defaults = {k: globals()[k] for k in overrides}
     for shape, rowsum in (("d128", "add"), ("d256", "add"), ("d64", "mfma")):
         SHAPE, ROWSUM = shape, rowsum
-        for k, v in overrides.items(): globals()[k] = v
+        for k, v in overrides.items():
+            if isinstance(v, dict): v = v.get(shape, rowsum if k == "ROWSUM" else defaults[k])   # {"ROWSUM": {"d128": "mfma"}}: one shape only
+            globals()[k] = v
         configure()
         out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fmha_fwd_loop16_%s.inc" % shape)
         txt = render()

@@ -354,7 +354,7 @@ class Checker:
         assert self.idx - last_mfma > 8
 
 
-@pytest.mark.parametrize("shape,rowsum,fold", [("d128", "mfma", False), ("d128", "add", True), ("d128", "add", False), ("d128", "dot", False),
+@pytest.mark.parametrize("shape,rowsum,fold", [("d128", "mfma", False), ("d128", "mfma", True), ("d128", "add", True), ("d128", "add", False), ("d128", "dot", False),
                                                ("d256", "add", True), ("d256", "add", False), ("d64", "mfma", True), ("d64", "mfma", False)])
 @pytest.mark.parametrize("n_tiles", [8, 12, 16, 32, 64])
 def test_loop_is_correct_symbolically(n_tiles, shape, rowsum, fold):
