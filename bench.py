@@ -64,6 +64,10 @@ WORKLOADS = {
     "cfg4_climb": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None, climb=True),
     "cfg4_climb_one_pass": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None, climb=True, one_pass=True),
     "cfg4_one_pass": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None, one_pass=True),
+    # cfk_set_option(CFK_OPT_FAST_E4M3_WEIGHTS, 1): e4m3 weights written as codes, without an exponential (an option: a
+    # fifth of the weights are then one e4m3 step off the correctly rounded one)
+    "cfg4_fast_weights": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None, fast_weights=True),
+    "d64_f8_fast_weights": dict(kind="fmha", dtype="f8", B=4, H=32, S=4096, D=64, scale=None, fast_weights=True),
     "d64_f16": dict(kind="fmha", dtype="f16", B=4, H=32, S=4096, D=64, scale=None),   # the reference sweep's head size 64
     "d64_f8": dict(kind="fmha", dtype="f8", B=4, H=32, S=4096, D=64, scale=None),
     "gemm_f32": dict(kind="gemm", dtype="f32", M=8192, N=8192, K=8192, max_steps=50),  # the CuTe example's type 1
@@ -78,6 +82,9 @@ NAMES = {
                   "every workgroup takes the second, max-tracking pass)",
     "cfg4_climb_one_pass": "... the same data with cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, 1): max-tracking pass only",
     "cfg4_one_pass": "fmha_fwd fp8-e4m3 B=4 H=16 S=4096 D=128 N(0,1) data with cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, 1)",
+    "cfg4_fast_weights": "fmha_fwd fp8-e4m3 B=4 H=16 S=4096 D=128 N(0,1) data with cfk_set_option(CFK_OPT_FAST_E4M3_WEIGHTS, 1): e4m3 weights "
+                         "written as codes without an exponential (not the default: a fifth of them one e4m3 step off)",
+    "d64_f8_fast_weights": "fmha_fwd fp8-e4m3 B=4 H=32 S=4096 D=64 with cfk_set_option(CFK_OPT_FAST_E4M3_WEIGHTS, 1)",
     "d64_f16": "fmha_fwd fp16 B=4 H=32 S=4096 D=64 non-causal (the reference sweep's problem at head size 64)",
     "d64_f8": "fmha_fwd fp8-e4m3 B=4 H=32 S=4096 D=64 non-causal, per-tensor amax scales, V [B,S,H,D]",
     "gemm_f32": "gemm fp32 M=N=K=8192 TN (fp32 MFMA: gfx950 has no tf32)",
@@ -154,6 +161,8 @@ def run_workload(pkg, name, steps, warmup):
     n = steps * 20 if name == "cfg1" else min(steps, w.get("max_steps", steps))
     if w.get("one_pass"):
         pkg.fmha.set_option(pkg.fmha.CFK_OPT_PREDICTABLE_LATENCY, 1)
+    if w.get("fast_weights"):
+        pkg.fmha.set_option(pkg.fmha.CFK_OPT_FAST_E4M3_WEIGHTS, 1)
     try:
         kernel = None
         if w["kind"] == "fmha":   # the instantiation the library launches for this call (cfk_fmha_forward_kernel)
@@ -163,6 +172,8 @@ def run_workload(pkg, name, steps, warmup):
     finally:
         if w.get("one_pass"):
             pkg.fmha.set_option(pkg.fmha.CFK_OPT_PREDICTABLE_LATENCY, 0)
+        if w.get("fast_weights"):
+            pkg.fmha.set_option(pkg.fmha.CFK_OPT_FAST_E4M3_WEIGHTS, 0)
     tflops = flop / (ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[w["dtype"]]
     return dict(workload=NAMES[name], ms_per_step=ms, wall_ms_per_step=wall_ms, tflops=tflops, flop_per_step=flop,

@@ -17,7 +17,7 @@
 namespace {
 
 thread_local char g_err[512] = "";
-std::atomic<int> g_predictable{0};
+std::atomic<int> g_predictable{0}, g_fast_e4m3{0};
 
 int fail(int code, const char *fmt, ...) {
   va_list ap;
@@ -93,6 +93,7 @@ int check_device() {
 
 namespace cfk {
 bool predictable_latency() { return g_predictable.load(std::memory_order_relaxed) != 0; }
+bool fast_e4m3_weights() { return g_fast_e4m3.load(std::memory_order_relaxed) != 0; }
 }  // namespace cfk
 
 extern "C" {
@@ -157,6 +158,7 @@ int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
   // 2, not 7, below a max, and only the first tile's).  Over the 4096 keys of the reference's own problem that is far
   // inside its error-percentage gate (fmha_forward.cu:638-639: 0.0000 % against 0.001 %); at 2048 keys the same measure
   // reads 0.0011 % for head dim 64, so key lengths below 4096 take the max-tracking pass only.
+  a.direct_p = g_fast_e4m3.load(std::memory_order_relaxed);
   a.track_only = cfk::predictable_latency() || (p->v_dtype == CFK_FP8_E4M3 && p->seqlen_kv < 4096) ? 1 : 0;
   hipError_t e;
   a.s_scale = p->dtype == CFK_FP16 ? p->softmax_scale : p->softmax_scale * p->q_descale * p->k_descale;
@@ -178,8 +180,9 @@ int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
 }
 
 int cfk_set_option(int32_t option, int32_t value) {
-  if (option != CFK_OPT_PREDICTABLE_LATENCY) return fail(CFK_ERR_INVALID_ARG, "unknown option %d", option);
-  g_predictable.store(value != 0, std::memory_order_relaxed);
+  if (option == CFK_OPT_PREDICTABLE_LATENCY) g_predictable.store(value != 0, std::memory_order_relaxed);
+  else if (option == CFK_OPT_FAST_E4M3_WEIGHTS) g_fast_e4m3.store(value != 0, std::memory_order_relaxed);
+  else return fail(CFK_ERR_INVALID_ARG, "unknown option %d", option);
   return CFK_OK;
 }
 

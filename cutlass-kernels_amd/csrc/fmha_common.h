@@ -22,10 +22,13 @@ struct FmhaArgs {
   int32_t v_layout;  // 0 = [B,S,H,D], 1 = [B,D,H,S]
   float tau;         // the softmax reference point moves when a tile's max exceeds it by more than this (log2 domain)
   int32_t track_only;  // no optimistic first pass over the keys (cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, 1))
+  int32_t direct_p;    // first pass with e4m3 P: codes without an exponential (cfk_set_option(CFK_OPT_FAST_E4M3_WEIGHTS, 1))
 };
 
 // cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, ...): also steers the choice of instantiation (fmha_fwd_kernel.h: select_tile)
 bool predictable_latency();
+// cfk_set_option(CFK_OPT_FAST_E4M3_WEIGHTS, ...): calls then launch the DirectCfg builds of the kernels with e4m3 P
+bool fast_e4m3_weights();
 
 struct FmhaPlan {
   int32_t block_m, block_n, lds_bytes, threads, grid;

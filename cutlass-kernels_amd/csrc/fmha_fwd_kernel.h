@@ -52,6 +52,7 @@
 //  * Workgroup ids are remapped so the query blocks of one head share an XCD's L2.
 #pragma once
 #include <cstdio>
+#include <cstring>
 #include <mutex>
 #include <type_traits>
 
@@ -69,6 +70,14 @@ typedef int int8v __attribute__((ext_vector_type(8)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int2v __attribute__((ext_vector_type(2)));
 
+// what a pass over the keys does: track the running row max tile by tile (value), build e4m3 weights without an
+// exponential (direct; only in a pass that does not track)
+template <bool TRACK_, bool DIRECT_>
+struct PassKind {
+  static constexpr bool value = TRACK_, direct = DIRECT_;
+  static_assert(!(TRACK_ && DIRECT_), "the direct codes belong to the pass with the fixed reference point");
+};
+
 template <int D_, int BN_, int NWAVES_, int WPE_, bool QK8_, bool PV8_, bool VT_ = false, bool TAP_S_ = false, int SUB_ = 1, int KPRE_ = 0,
           bool M16_ = false, bool ASM_ = false>
 struct FmhaCfg {
@@ -82,6 +91,7 @@ struct FmhaCfg {
   static constexpr int NSLOT_V = 2 * SUB;                       // ... and of V
   static constexpr int WPE = WPE_;                              // waves per SIMD the register budget is sized for
   static constexpr bool QK8 = QK8_, PV8 = PV8_;                 // e4m3 (true) or fp16 (false) operands of GEMM-I / II
+  static constexpr bool DIRECT = false;                         // (DirectCfg below)
   static constexpr bool VT = VT_;                               // V given pre-transposed, [B,D,H,S] (e4m3 only)
   static constexpr bool TAP_S = TAP_S_;                         // also write the pre-softmax scores (debug build)
   static constexpr int T = NWAVES * 64;
@@ -368,7 +378,32 @@ fmha_fwd_kernel(const FmhaArgs a) {
   };
   // P = exp2(c*S - m_ref); row sum in fp32 before the down-cast (online_softmax.h:173-206); cast in the B-operand
   // register order of the second GEMM
-  auto softmax_exp = [&](const f32x16 (&sacc)[KB], PReg (&pb)[PS]) __attribute__((always_inline)) {
+  // DIRECT (DirectCfg builds: first pass with e4m3 P and the row sum on the matrix pipe, launched for callers that set
+  // CFK_OPT_FAST_E4M3_WEIGHTS): the e4m3 code of a weight is built without an exponential.  Read as an integer, the code of a positive e4m3 number is 8 (log2 of it + 7) with the mantissa
+  // interpolated linearly, so sat_u8(rne(8 (c S - m) + 56 - 0.46)) is exp2(c S - m) rounded to e4m3 up to that
+  // interpolation (0.46: its mean; a fifth of the codes differ from the correctly rounded one, by one step; tests/
+  // test_oracle.py pins the formula against the codec): one multiply-add and one v_cvt_pk_u8_f32 per score (4 issue
+  // cycles each) in place of multiply-add, v_exp_f32 (8) and half a v_cvt_pk_fp8_f32 (8).  The conversion saturates at
+  // 255: code 0x7F is NaN and reaches the row sum through the MFMA, codes from 0x80 on (negative numbers) are caught by
+  // the OR of all P registers in p_flags.
+  constexpr bool DIRECT_OK = C::DIRECT;
+  static_assert(!C::DIRECT || (PV8 && MFMA_SUM), "direct codes: e4m3 P with the row sum on the matrix pipe");
+  uint32_t p_flags = 0;
+  auto softmax_exp = [&](auto direct, const f32x16 (&sacc)[KB], PReg (&pb)[PS]) __attribute__((always_inline)) {
+    if constexpr (decltype(direct)::value && DIRECT_OK) {
+      const float c8 = 8.0f * c_log2, m8 = 8.0f * m_ref - 55.54f;
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          uint32_t code = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(sacc[kb][4 * w], c8, -m8), 0, 0u);
+#pragma unroll
+          for (int t = 1; t < 4; ++t) code = __builtin_amdgcn_cvt_pk_u8_f32(__builtin_fmaf(sacc[kb][4 * w + t], c8, -m8), t, code);
+          p_flags |= code;
+          pb[kb / 2][(kb % 2) * 4 + w] = (int)code;
+        }
+      return;
+    }
     float rs = 0.f;
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
@@ -476,16 +511,17 @@ fmha_fwd_kernel(const FmhaArgs a) {
     if constexpr (FENCED) __builtin_amdgcn_sched_barrier(0);
   };
   // qk(next) and the exponentials of the current tile, in the order of the build
-  auto qk_and_exp = [&](auto has_next, int k_stage, f32x16 (&s_nxt)[KB], f32x16 (&s_cur)[KB], PReg (&pb)[PS]) __attribute__((always_inline)) {
+  auto qk_and_exp = [&](auto track, auto has_next, int k_stage, f32x16 (&s_nxt)[KB], f32x16 (&s_cur)[KB], PReg (&pb)[PS]) __attribute__((always_inline)) {
     constexpr bool HAS_NEXT = decltype(has_next)::value;
+    constexpr std::integral_constant<bool, decltype(track)::direct> direct{};
     if constexpr (EXP_FIRST) {
-      softmax_exp(s_cur, pb);
+      softmax_exp(direct, s_cur, pb);
       fence();
       if (HAS_NEXT) qk(k_stage, s_nxt);
     } else {
       if (HAS_NEXT) qk(k_stage, s_nxt);
       fence();
-      softmax_exp(s_cur, pb);
+      softmax_exp(direct, s_cur, pb);
     }
     fence();
   };
@@ -501,7 +537,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
     load_k(j + 2 < n_tiles ? j + 2 : n_tiles - 1, P);
     load_v(j + 1 < n_tiles ? j + 1 : n_tiles - 1, P ^ 1);
     PReg pb[PS];
-    qk_and_exp(has_next, P ^ 1, s_nxt, s_cur, pb);
+    qk_and_exp(track, has_next, P ^ 1, s_nxt, s_cur, pb);
     pv(P * C::V_TILE, pb);
     if (TRACK && HAS_NEXT) row_max_and_rescale(s_nxt, j + 1);
     wait_lds_dma();   // this wave's copies have landed ...
@@ -521,7 +557,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
     load_k(t0 + 4 < t_max ? t0 + 4 : t_max, (2 * P) % 4);
     {
       PReg pb[PS];
-      qk_and_exp(std::true_type{}, (2 * P + 1) % 4, s_b, s_a, pb);
+      qk_and_exp(track, std::true_type{}, (2 * P + 1) % 4, s_b, s_a, pb);
       pv(((2 * P) % 4) * C::V_TILE, pb);
       if (TRACK) row_max_and_rescale(s_b, t0 + 1);
     }
@@ -529,7 +565,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
     load_v(t0 + 3 < t_max ? t0 + 3 : t_max, (2 * P + 3) % 4);
     {
       PReg pb[PS];
-      qk_and_exp(std::integral_constant<bool, !LAST>{}, (2 * P + 2) % 4, s_a, s_b, pb);
+      qk_and_exp(track, std::integral_constant<bool, !LAST>{}, (2 * P + 2) % 4, s_a, s_b, pb);
       pv(((2 * P + 1) % 4) * C::V_TILE, pb);
       if (TRACK && !LAST) row_max_and_rescale(s_a, t0 + 2);
     }
@@ -550,7 +586,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
     if (HAS_NEXT) qk((J4 + 1) % 4, s_nxt, true);
     load_k(j + 3 < n_tiles ? j + 3 : n_tiles - 1, (J4 + 3) % 4);
     load_v(j + 1 < n_tiles ? j + 1 : n_tiles - 1, P ^ 1);
-    softmax_exp(s_cur, pb);
+    softmax_exp(std::integral_constant<bool, decltype(track)::direct>{}, s_cur, pb);
     pv(P * C::V_TILE, pb);
     if (HAS_NEXT) {
       prefetch_k((J4 + 2) % 4);
@@ -657,12 +693,12 @@ fmha_fwd_kernel(const FmhaArgs a) {
   // (fp16 P gains nothing from the first pass -- its row max hides behind the second GEMM's MFMAs -- and skips it.)
   bool redo = !PV8 || C::TAP_S || a.row_max != nullptr || a.row_sum != nullptr || !(kTau > 0.f) || a.track_only != 0;
   if (!redo) {
-    pass(integral_constant<bool, false>{});
+    pass(PassKind<false, DIRECT_OK>{});
     const float l_chk = MFMA_SUM ? l_acc[0] : l_run;
-    const bool bad = !(__builtin_fabsf(oacc[0][0]) < 3.0e38f) || !(l_chk < 3.0e38f);
+    const bool bad = !(__builtin_fabsf(oacc[0][0]) < 3.0e38f) || !(l_chk < 3.0e38f) || (p_flags & 0x80808080u) != 0;
     redo = __syncthreads_or(bad) != 0;
   }
-  if (redo) pass(integral_constant<bool, true>{});
+  if (redo) pass(PassKind<true, false>{});
 
   // ---- epilogue: O = out_scale * O / l (online_softmax.h:59-85), fp16, [B,S,H,D]; a lane holds 4 consecutive d
   const float l_tot = MFMA_SUM ? l_acc[0] : l_run + __shfl_xor(l_run, 32, 64);
@@ -718,6 +754,15 @@ template <class C>
 __global__ void __launch_bounds__(C::T) fmha_fwd_kernel_ks(const FmhaArgs a);
 
 // the kernel an instantiation runs
+// The same build with the e4m3 weights of the first pass written as codes, without an exponential (see softmax_exp in
+// fmha_fwd_kernel and gen_fmha_loop8.py): what a call gets under cfk_set_option(CFK_OPT_FAST_E4M3_WEIGHTS, 1).
+template <class C>
+struct DirectCfg : C {
+  static constexpr bool DIRECT = true;
+};
+template <class C>
+constexpr bool has_direct_build = C::PV8 && C::D <= 128 && !C::TAP_S && !C::KSPLIT;
+
 template <class C>
 constexpr auto fmha_kernel_of() {
   if constexpr (C::KSPLIT) return &fmha_fwd_kernel_ks<C>;
@@ -744,6 +789,10 @@ hipError_t prepare_fmha_cfg() {
   static hipError_t status = hipSuccess;
   std::call_once(once, [] {
     status = hipFuncSetAttribute((const void *)fmha_kernel_of<C>(), hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if constexpr (has_direct_build<C>) {
+      const hipError_t e = hipFuncSetAttribute((const void *)fmha_kernel_of<DirectCfg<C>>(), hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+      if (status == hipSuccess) status = e;
+    }
   });
   return status;
 }
@@ -754,6 +803,12 @@ hipError_t launch_fmha_cfg(const FmhaArgs &a, hipStream_t s) {
   if (e != hipSuccess) return e;
   const int items = a.B * a.H * (a.Sq / C::BM);
   const int grid = C::ASM ? persistent_grid(items) : items;
+  if constexpr (has_direct_build<C>) {
+    if (a.direct_p != 0) {
+      hipLaunchKernelGGL(fmha_kernel_of<DirectCfg<C>>(), dim3(grid), dim3(C::T), C::LDS_BYTES, s, a);
+      return hipGetLastError();
+    }
+  }
   hipLaunchKernelGGL(fmha_kernel_of<C>(), dim3(grid), dim3(C::T), C::LDS_BYTES, s, a);
   return hipGetLastError();
 }
@@ -773,6 +828,9 @@ void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
   snprintf(p->kernel, sizeof p->kernel, "%s<%d,%d,%d,%d,%d,%d,%d,%d,%d,%d,%d,%d>",
            C::ASM ? (C::QK8 ? "fmha_fwd_kernel8p" : "fmha_fwd_kernel16p") : C::M16 ? "fmha_fwd_kernel16" : "fmha_fwd_kernel", C::D, C::BN, C::NWAVES, C::WPE,
            (int)C::QK8, (int)C::PV8, (int)C::VT, (int)C::TAP_S, C::SUB, C::KPRE, (int)C::M16, (int)C::ASM);
+  if constexpr (has_direct_build<C>) {
+    if (fast_e4m3_weights()) strncat(p->kernel, "/direct", sizeof p->kernel - strlen(p->kernel) - 1);   // the DirectCfg build
+  }
 }
 
 // ---- tile selection.  The reference fixes its tile at compile time (-DQBLKSIZE / -DKBLKSIZE,

@@ -2,8 +2,8 @@
 """Generator of the hand-scheduled main loop of the e4m3 FMHA forward kernel (fmha_fwd_kernel8p.h): head dim 128, 256
 query rows per workgroup (8 waves x 32 rows, two waves per SIMD), 64-key tiles, V in [B,S,H,D].
 
-    python3 gen_fmha_loop8.py            # rewrites fmha_fwd_loop8_d128.inc beside this file
-    python3 gen_fmha_loop8.py --check    # exit status 1 if that file is not what the generator produces
+    python3 gen_fmha_loop8.py            # rewrites fmha_fwd_loop8_d128.inc and fmha_fwd_loop8_d128_direct.inc beside this file
+    python3 gen_fmha_loop8.py --check    # exit status 1 if those files are not what the generator produces
 
 Why: this kernel is bound by instruction issue, not by the matrix pipe.  Measured with register-only loops (two waves per
 SIMD, cycles of the SIMD per v_mfma_f32_32x32x64_f8f6f4, 64.0 with nothing else): twelve ordinary vector instructions or
@@ -57,12 +57,23 @@ T = 9                                    # MFMA places per tile
 
 O0, SA0, SB0, Q0, P0, RING0 = 192, 128, 160, 112, 96, 48
 LACC0, ONES0, KRD0, VRD0, GOK, GOV, MREF, QOFF = 44, 36, 24, 28, 32, 33, 34, 35
+FLAGS = 80         # DIRECT: OR of all P registers of the item (a byte with bit 7 set is a weight beyond the e4m3 range)
 LOW = 24
 RING = 4
 LOOKAHEAD = 3      # fragments requested ahead of use
 HOLD = 2           # MFMAs of a super-step issued behind its barrier
 VALU_START = 3.0   # place (within tile t's period) where softmax(t+1) starts
 MIN_MFMA_TO_VALU = 20   # instructions between an MFMA and the first vector instruction that reads its result
+# DIRECT: the e4m3 codes of the weights are built without an exponential.  The code of a positive e4m3 number, read as
+# an integer, is 8 (log2 of the number + 7) with the mantissa interpolated linearly (exact at the powers of two), so
+# P = sat_u8(rne(8 (c S - m) + 56 - 0.46)) is exp2(c S - m) rounded to e4m3 up to that interpolation (0.46: its mean, so
+# that the codes are unbiased; a fifth of them differ from the correctly rounded code, by one step).  The caller passes
+# c_loop = 8 c and m_loop = 8 m - 55.54 (otherwise c and m); per score one multiply-add and one v_cvt_pk_u8_f32 (4 issue cycles
+# each, measured) replace multiply-add, v_exp_f32 (8) and half a v_cvt_pk_fp8_f32 (8).  The conversion saturates at 255:
+# code 0x7F is NaN and reaches the row sum through the MFMA, codes from 0x80 on (negative numbers) are caught by the
+# OR of all P registers in v[FLAGS].  Both forms are generated; the kernel takes this one for callers that set
+# CFK_OPT_FAST_E4M3_WEIGHTS (a fifth of the weights one code off is a price the default does not pay).
+DIRECT = False
 ABLATE = set(os.environ.get("LOOP8_ABLATE", "").split(",")) - {""}
 
 
@@ -108,6 +119,10 @@ def softmax_ops(t):
             s = s_reg(t, kb) + 4 * w
             p = p_reg(t) + 4 * kb + w
             for i in range(4): ops.append(("v_fma_f32 v%d, v%d, %%[c], -v%d" % (s + i, s + i, MREF), 1))
+            if DIRECT:
+                for i in range(4): ops.append(("v_cvt_pk_u8_f32 v%d, v%d, %d, %s" % (p, s + i, i, "v%d" % p if i else "0"), 1))
+                if w % 2: ops.append(("v_or3_b32 v%d, v%d, v%d, v%d" % (FLAGS, FLAGS, p - 1, p), 1))
+                continue
             for i in range(4): ops.append(("v_exp_f32 v%d, v%d" % (s + i, s + i), 2))
             ops.append(("v_cvt_pk_fp8_f32 v%d, v%d, v%d" % (p, s, s + 1), 2))
             ops.append(("v_cvt_pk_fp8_f32 v%d, v%d, v%d op_sel:[0,0,1]" % (p, s + 2, s + 3), 2))
@@ -197,6 +212,7 @@ def schedule(n_tiles):
     cur.append("s_nop 7"); cur.append("s_nop 7"); cur.append("s_nop 7")   # MFMA results of the caller's S(0) are read by vector instructions
     for r in range(O0, O0 + 64): cur.append("v_mov_b32 v%d, 0" % r)
     for r in range(LACC0, LACC0 + 4): cur.append("v_mov_b32 v%d, 0" % r)
+    if DIRECT: cur.append("v_mov_b32 v%d, 0" % FLAGS)
     if "reads" in ABLATE:
         for r in range(RING0, RING0 + 8 * RING): cur.append("v_mov_b32 v%d, 0" % r)
     request(0, LOOKAHEAD)
@@ -254,11 +270,15 @@ def render():
     sa1 (in, clobbered: S(0) of key blocks 0, 1), qv (in: this item's Q; out: the next item's); f32x4 lacc (out: the row
     sum, complete in every lane); int8v ones (the 0/1 operand); uint64_t kptr, vptr (in: this item's K tile 3 / V tile
     2; out: the same of the next item), kn, vn, qn (the next item's K, V and this wave's Q rows); uint32_t nloop,
-    k_rd[4], v_rd[4], goff_k, goff_v, qoff, lds_wave, tile_stride; float m_ref, c_log2."""
+    k_rd[4], v_rd[4], goff_k, goff_v, qoff, lds_wave, tile_stride; float m_loop, c_loop; with DIRECT also uint32_t p_flags
+    (out) and constexpr bool kDirect."""
     head, body, tail = folded()
     L = []
     L.append("// GENERATED by gen_fmha_loop8.py -- do not edit.  The hand-scheduled main loop of fmha_fwd_kernel8p (e4m3, head dim")
     L.append("// 128, 256 x 128): %d + %d (loop) + %d instructions." % (len(head), len(body), len(tail)))
+    L.append("// The weights are built as e4m3 codes without an exponential: c_loop = 8 c, m_loop = 8 m - 55.54, p_flags = OR of all P (true);")
+    L.append("// or with v_exp_f32 and v_cvt_pk_fp8_f32: c_loop = c, m_loop = m (false)")
+    L.append("static_assert(kDirect == %s, \"the caller passes the scale and the reference point in the form this loop takes\");" % ("true" if DIRECT else "false"))
     L.append("asm volatile(")
     def emit(ins): L.append('    "%s\\n"' % ins)
     for i in head: emit(i)
@@ -271,24 +291,35 @@ def render():
     emit("s_cbranch_scc1 1b")
     emit("2:")
     for i in tail: emit(i)
-    L.append('    : "={v[192:207]}"(o0), "={v[208:223]}"(o1), "={v[224:239]}"(o2), "={v[240:255]}"(o3), "={v[44:47]}"(lacc),')
+    L.append('    : "={v[192:207]}"(o0), "={v[208:223]}"(o1), "={v[224:239]}"(o2), "={v[240:255]}"(o3), "={v[44:47]}"(lacc),%s' % (' "={v%d}"(p_flags),' % FLAGS if DIRECT else ""))
     L.append('      "+{v[128:143]}"(sa0), "+{v[144:159]}"(sa1), "+{v[112:127]}"(qv), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), [nloop] "+s"(nloop)')
     ins = ['"{v[36:43]}"(ones)', '"{v%d}"(qoff)' % QOFF, '[kn] "s"(kn)', '[vn] "s"(vn)', '[qn] "s"(qn)']
     ins += ['"{v%d}"(k_rd[%d])' % (KRD0 + i, i) for i in range(4)] + ['"{v%d}"(v_rd[%d])' % (VRD0 + i, i) for i in range(DB)]
-    ins += ['"{v%d}"(goff_k)' % GOK, '"{v%d}"(goff_v)' % GOV, '"{v%d}"(m_ref)' % MREF]
-    ins += ['[c] "s"(c_log2)', '[ldsw] "s"(lds_wave)', '[stride] "s"(tile_stride)']
+    ins += ['"{v%d}"(goff_k)' % GOK, '"{v%d}"(goff_v)' % GOV, '"{v%d}"(m_loop)' % MREF]
+    ins += ['[c] "s"(c_loop)', '[ldsw] "s"(lds_wave)', '[stride] "s"(tile_stride)']
     L.append("    : " + ", ".join(ins))
     used = set(range(O0, O0 + 64)) | set(range(SA0, SA0 + 32)) | set(range(Q0, Q0 + 16)) | set(range(LOW, LACC0 + 4))
-    clob = ['"memory"', '"scc"', '"m0"'] + ['"v%d"' % r for r in range(LOW, 256) if r not in used]
+    if DIRECT: used.add(FLAGS)
+    # (registers the loop never names stay the compiler's: values it keeps across the statement need not be spilled)
+    import re
+    named = set()
+    for ins in head + body + tail:
+        for m in re.finditer(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b", ins):
+            named |= set(range(int(m.group(1)), int(m.group(2)) + 1)) if m.group(1) else {int(m.group(3))}
+    clob = ['"memory"', '"scc"', '"m0"'] + ['"v%d"' % r for r in range(LOW, 256) if r not in used and r in named]
     L.append("    : " + ", ".join(clob) + ");")
     return "\n".join(L) + "\n"
 
 
 if __name__ == "__main__":
     for k, v in json.loads(os.environ.get("LOOP8_SET", "{}")).items(): globals()[k] = v
-    out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "fmha_fwd_loop8_d128.inc")
-    txt = render()
-    if "--check" in sys.argv:
-        sys.exit(0 if os.path.exists(out) and open(out).read() == txt else 1)
-    open(out, "w").write(txt)
-    print("wrote", out, len(txt.splitlines()), "lines")
+    stale = False
+    for DIRECT, name in ((False, "fmha_fwd_loop8_d128.inc"), (True, "fmha_fwd_loop8_d128_direct.inc")):
+        out = os.path.join(os.path.dirname(os.path.abspath(__file__)), name)
+        txt = render()
+        if "--check" in sys.argv:
+            stale = stale or not (os.path.exists(out) and open(out).read() == txt)
+        else:
+            open(out, "w").write(txt)
+            print("wrote", out, len(txt.splitlines()), "lines")
+    sys.exit(1 if stale else 0)

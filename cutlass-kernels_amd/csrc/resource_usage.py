@@ -34,9 +34,10 @@ def short_name(d):
     if m: return m.group(1) + "<" + m.group(2).replace("Lb0E", "0,").replace("Lb1E", "1,").replace("Li4E", "4").rstrip(",") + ">"
     d = re.sub(r"^void ", "", d).replace("(anonymous namespace)::", "")
     d = re.sub(r"\(.*\)$", "", d)
-    d = d.replace("cfk::", "").replace("FmhaCfg<", "").replace("KsCfg<", "").replace(">>", ">").replace(">>", ">")
+    direct = "DirectCfg<" in d     # the build with e4m3 weights written as codes: shown as <...>/direct
+    d = d.replace("cfk::", "").replace("DirectCfg<", "").replace("FmhaCfg<", "").replace("KsCfg<", "").replace(">>", ">").replace(">>", ">")
     d = d.replace("false", "0").replace("true", "1").replace(" ", "")
-    return re.sub(r">+$", ">", d)
+    return re.sub(r">+$", ">", d) + ("/direct" if direct else "")
 
 
 def compile_one(src):

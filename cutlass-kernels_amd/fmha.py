@@ -23,6 +23,7 @@ CFK_V_BDHS = 1
 CFK_GEMM_TN = 0
 CFK_GEMM_NN = 1
 CFK_OPT_PREDICTABLE_LATENCY = 1
+CFK_OPT_FAST_E4M3_WEIGHTS = 2
 
 
 class CfkError(RuntimeError):
@@ -105,7 +106,7 @@ def init() -> None:
 
 
 def set_option(option: int, value: int) -> None:
-    """``cfk_set_option``: process-wide options, e.g. ``CFK_OPT_PREDICTABLE_LATENCY``."""
+    """``cfk_set_option``: process-wide options (``CFK_OPT_PREDICTABLE_LATENCY``, ``CFK_OPT_FAST_E4M3_WEIGHTS``)."""
     _check(lib().cfk_set_option(option, value))
 
 

@@ -159,7 +159,18 @@ typedef enum cfk_option {
    * 128 on big problems.  On scores that climb along the key axis that costs up to twice the time.  With this option
    * every call takes the max-tracking path from the start: the same results to rounding, a run time that does not
    * depend on the data (a few per cent slower on ordinary data).  0 (default): two passes where they pay. */
-  CFK_OPT_PREDICTABLE_LATENCY = 1
+  CFK_OPT_PREDICTABLE_LATENCY = 1,
+  /* 1: e4m3 weights without an exponential.  In the first of the two passes above, kernels with e4m3 P (head dims 64
+   * and 128) then build the e4m3 code of a weight directly: read as an integer, the code of a positive e4m3 number is
+   * 8 (log2 of it + 7) with the mantissa interpolated linearly, so sat_u8(round(8 (c s - m) + 55.54)) is exp2(c s - m)
+   * rounded to e4m3 up to that interpolation -- one multiply-add and one conversion per score in place of multiply-add,
+   * exponential and conversion: +11 % on B=4 H=16 S=4096 D=128, +27 % at head dim 64.  A fifth of the weights then
+   * differ from the correctly rounded code by one step: on N(0,1) data the rms error of O against the fp32 reference
+   * grows from 6.8e-4 to 8.1e-4 and the share of elements that fail the reference's own check (|d| > 5e-3 and more
+   * than 10 % relative, src/fmha-pipeline/fmha_forward.cu:638-639) from 0-1e-4 % to 1e-4-6e-4 % with excursions above
+   * its limit of 1e-3 % -- which is why this is an option.  The max-tracking pass always takes the exponential.
+   * 0 (default): exponential and conversion everywhere. */
+  CFK_OPT_FAST_E4M3_WEIGHTS = 2
 } cfk_option;
 int cfk_set_option(int32_t option, int32_t value);
 

@@ -146,5 +146,17 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
         assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128) == "fmha_fwd_kernel<128,64,8,2,1,1,0,0,2,0,0,0>"
     finally:
         f.set_option(f.CFK_OPT_PREDICTABLE_LATENCY, 0)
+    # e4m3 weights without an exponential: the same choice of tile, the DirectCfg build of it; kernels without e4m3 P
+    # have no such build
+    f.set_option(f.CFK_OPT_FAST_E4M3_WEIGHTS, 1)
+    try:
+        assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128) == "fmha_fwd_kernel8p<128,64,8,2,1,1,0,0,2,0,0,1>/direct"
+        assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 4, 32, 4096, 4096, 64) == "fmha_fwd_kernel<64,64,4,3,1,1,0,0,1,0,0,0>/direct"
+        assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 2048, 2048, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
+        assert "/direct" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128, v_dtype=f.CFK_FP16)
+        assert "/direct" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 2, 8, 4096, 4096, 256)
+    finally:
+        f.set_option(f.CFK_OPT_FAST_E4M3_WEIGHTS, 0)
+    assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128) == "fmha_fwd_kernel8p<128,64,8,2,1,1,0,0,2,0,0,1>"
     with pytest.raises(pkg.CfkError):
         f.set_option(99, 1)

@@ -439,3 +439,64 @@ def test_predictable_latency_option_takes_the_tracked_pass():
     assert np.array_equal(o_opt, o_taps)
     ref = oracle.attention_f32(qf, kf, vf)["O"]
     assert max_abs(o_default, ref) <= TOL_FP8 and max_abs(o_opt, ref) <= TOL_FP8
+
+
+# ---- cfk_set_option(CFK_OPT_FAST_E4M3_WEIGHTS, 1): the first pass writes the e4m3 codes of the weights without an
+# exponential (the DirectCfg builds).  Same gate as everything else here; what is looser than with the default is
+# the reference's own error percentage, which is why this is an option (the header says by how much).
+@pytest.fixture
+def fast_weights():
+    f = pkg.fmha
+    f.set_option(f.CFK_OPT_FAST_E4M3_WEIGHTS, 1)
+    try:
+        yield f
+    finally:
+        f.set_option(f.CFK_OPT_FAST_E4M3_WEIGHTS, 0)
+
+
+@pytest.mark.parametrize("B,S,H,D,v_layout", [(4, 4096, 16, 128, None), (1, 4096, 4, 128, None), (2, 4096, 8, 64, None),
+                                              (1, 4096, 8, 64, "bdhs"), (1, 4096, 4, 128, "bdhs")])
+def test_fast_e4m3_weights_parity(fast_weights, B, S, H, D, v_layout):
+    import torch
+    f = fast_weights
+    name = f.fmha_forward_kernel(f.CFK_FP8_E4M3, B, H, S, S, D, v_layout=f.CFK_V_BDHS if v_layout else f.CFK_V_BSHD)
+    assert name.endswith("/direct"), name
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    (qc, qs, qf), (kc, ks, kf), (vc, vs, vf) = _quant(q), _quant(k), _quant(v)
+    kw = dict(q_descale=qs, k_descale=ks, v_descale=vs)
+    vdev = to_dev(np.ascontiguousarray(vc.transpose(0, 3, 2, 1))) if v_layout else to_dev(vc)
+    if v_layout: kw["v_layout"] = f.CFK_V_BDHS
+    fast = pkg.fmha_forward(to_dev(qc), to_dev(kc), vdev, **kw)
+    torch.cuda.synchronize()
+    f.set_option(f.CFK_OPT_FAST_E4M3_WEIGHTS, 0)
+    exact = pkg.fmha_forward(to_dev(qc), to_dev(kc), vdev, **kw)
+    torch.cuda.synchronize()
+    fast, exact = fast.float().cpu().numpy(), exact.float().cpu().numpy()
+    pairs = sorted({(0, 0), (B - 1, H - 1)})
+    ref = oracle.attention_f32(qf, kf, vf, bh_pairs=pairs)["O"]
+    sel = ~np.isnan(ref)
+    e_fast, e_exact = np.abs(fast[sel] - ref[sel]), np.abs(exact[sel] - ref[sel])
+    rms = lambda e: float(np.sqrt((e.astype(np.float64) ** 2).mean()))
+    print(f"e4m3 fast weights {name}: max-abs {e_fast.max():.3e} (default {e_exact.max():.3e}), rms {rms(e_fast):.3e} ({rms(e_exact):.3e})")
+    assert not np.isnan(fast).any() and e_fast.max() <= TOL_FP8
+    assert not np.array_equal(fast, exact)                 # the option did change the kernel that ran ...
+    assert rms(e_fast) <= 1.35 * rms(e_exact)              # ... by about what a fifth of the codes one step off costs
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_fast_e4m3_weights_second_pass(fast_weights, D):
+    # weights beyond the e4m3 range come out of the conversion as 0x7F (NaN, seen in the row sum) or with bit 7 set (seen
+    # in the OR of the P registers): climbing keys, then a single row whose score leaves the range by a wide margin
+    import torch
+    _climb_case(1, 256, 2, D, 4096)
+    if D == 128: _climb_case(4, 4096, 16, 128, 4096, ramp=1.5, spike=1.0)   # the hand-scheduled build; some workgroups only
+    B, S, H, Skv = 1, 256, 2, 4096
+    q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=Skv)
+    q[0, 77, 1] = 6.0 * k[0, 1000, 1]
+    (qc, qs, qf), (kc, ks, kf), (vc, vs, vf) = _quant(q), _quant(k), _quant(v)
+    o = pkg.fmha_forward(to_dev(qc), to_dev(kc), to_dev(vc), q_descale=qs, k_descale=ks, v_descale=vs)
+    torch.cuda.synchronize()
+    got = o.float().cpu().numpy()
+    ref = oracle.attention_f32(qf, kf, vf)["O"]
+    assert max_abs(got[0, 77, 1], vf[0, 1000, 1]) <= TOL_FP8
+    assert not np.isnan(got).any() and max_abs(got, ref) <= TOL_FP8

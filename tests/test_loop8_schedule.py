@@ -58,7 +58,7 @@ class Checker:
         self.inflight = []    # copies issued since the last barrier: (kind, slot, tile)
         self.seg_reads = set()
         self.waited_all = False
-        self.n_mfma = self.n_qk = 0
+        self.n_mfma = self.n_qk = self.n_flagged = 0
         for s in range(g.KS):
             for i in range(8): self.put(g.q_reg(s) + i, ("Q", s, i), FOREVER, "init")
         self.put(g.MREF, ("m",), FOREVER, "init")
@@ -164,8 +164,27 @@ class Checker:
             elif op == "v_exp_f32":
                 d, s_ = int(a[0][1:]), int(a[1][1:])
                 tag = self.get(s_, "valu")
-                assert d == s_ and tag[0] == "X", ins
+                assert not g.DIRECT and d == s_ and tag[0] == "X", ins
                 self.put(d, ("E",) + tag[1:], 1, "trans")
+            elif op == "v_cvt_pk_u8_f32":   # byte `byte` of a P register: the e4m3 code of one weight, straight from X
+                d, s_, byte, src2 = int(a[0][1:]), int(a[1][1:]), int(a[2]), a[3]
+                tag = self.get(s_, "valu")
+                assert g.DIRECT and tag[0] == "X", ins
+                t, kb, e = tag[1], tag[2], tag[3]
+                w = e // 4
+                assert e % 4 == byte and d == g.p_reg(t) + 4 * kb + w, ins
+                if byte == 0: assert src2 == "0", ins
+                else: assert src2 == "v%d" % d and self.get(d, "valu") == ("Pb", t, kb, w, byte - 1), ins
+                if byte < 3: self.put(d, ("Pb", t, kb, w, byte), 1, "valu")
+                else: self.put(d, ("P", t, kb, w), g.DB + 2, "valu")   # four P.V MFMAs, the row sum, the flags
+            elif op == "v_or3_b32":         # every P register goes into the overflow flags exactly once
+                d = int(a[0][1:])
+                assert g.DIRECT and d == g.FLAGS and a[1] == "v%d" % d, ins
+                assert self.get(d, "valu")[0] in ("zero", "flags")
+                ta, tb = self.get(int(a[2][1:]), "valu"), self.get(int(a[3][1:]), "valu")
+                assert ta[0] == "P" and tb[0] == "P" and ta[1:3] == tb[1:3] and ta[3] % 2 == 0 and tb[3] == ta[3] + 1, ins
+                self.n_flagged += 2
+                self.put(d, ("flags",), FOREVER, "valu")
             elif op == "v_cvt_pk_fp8_f32":
                 high = a[-1].endswith("op_sel:[0") or "op_sel" in rest
                 d = int(a[0][1:])
@@ -287,6 +306,7 @@ class Checker:
         for db in range(g.DB):
             for i in range(16): assert self.v[g.o_reg(db) + i].tag == ("O", db, n, i)
         for i in range(4): assert self.v[g.LACC0 + i].tag == ("lacc", n, i)
+        if g.DIRECT: assert self.n_flagged == 4 * g.KB * n and self.v[g.FLAGS].tag == ("flags",)
         assert self.n_mfma == g.KB * g.KS * (n - 1) + (g.DB + 1) * n
         # the next work item: its first three K and two V tiles are on their way into slots 0-2 / 0-1, its Q is in the Q
         # registers, and everything has been waited for
@@ -300,9 +320,11 @@ class Checker:
         assert self.idx - last_mfma > g.MIN_MFMA_TO_VALU
 
 
+@pytest.mark.parametrize("direct", [True, False])
 @pytest.mark.parametrize("n_tiles", [8, 12, 16, 32, 64, 128])
-def test_loop_is_correct_symbolically(n_tiles):
+def test_loop_is_correct_symbolically(n_tiles, direct):
     g = _gen()
+    g.DIRECT = direct
     c = Checker(g, n_tiles)
     c.run(g.program(n_tiles))
     c.finish()

@@ -258,3 +258,29 @@ def test_online_tiled_softmax_equals_direct(bN):
     # with P rounded to fp16 the error stays far inside the 2e-3 gate
     o16, _, _ = oracle.online_softmax_tiled(q, k, v, bN, scale * oracle.LOG2E, p_cast="f16")
     assert np.max(np.abs(o16 - r["O"][0, :, 0])) < 1e-3
+
+
+def test_e4m3_codes_of_an_exponential_built_without_an_exponential():
+    # The hand-scheduled e4m3 loop (fmha_fwd_kernel8p.h, gen_fmha_loop8.py: DIRECT) writes the weight exp2(x) as the byte
+    # sat_u8(rne(8 x + 55.54)): read as an integer, a positive e4m3 code is 8 (log2 + 7) with the mantissa interpolated
+    # linearly, and 0.46 = 56 - 55.54 is the mean distance of that interpolation from the exponential.  Pinned here
+    # against the codec: never more than one code away from the correctly rounded weight, the same code for most x,
+    # unbiased, and everything beyond the e4m3 range lands on NaN (0x7F) or on a code with bit 7 set, which is what the
+    # kernel's overflow vote looks for.
+    x = np.linspace(-6.0, 8.80, 200001)                      # the normal numbers: 2^-6 .. 446
+    code = np.clip(np.rint(8.0 * x + 55.54), 0, 255).astype(np.int64)
+    exact = oracle.e4m3_encode(np.exp2(x)).astype(np.int64)
+    assert np.abs(code - exact).max() == 1
+    assert (code == exact).mean() > 0.75
+    rel = oracle.e4m3_decode(code).astype(np.float64) / np.exp2(x) - 1.0
+    rel_exact = oracle.e4m3_decode(exact).astype(np.float64) / np.exp2(x) - 1.0
+    assert abs(rel.mean()) < 2e-3 and np.abs(rel).max() < 0.10          # (correct rounding: max 6.25 %)
+    assert np.sqrt((rel ** 2).mean()) < 1.3 * np.sqrt((rel_exact ** 2).mean())
+    # below the normal range the codes run out linearly (code 0 from x = -7 on): weights under 2^-6, 0.4 % of the row max
+    small = np.clip(np.rint(8.0 * np.linspace(-12, -6, 1001) + 55.54), 0, 255).astype(np.int64)
+    assert small.max() <= 8 and small.min() == 0 and np.all(np.diff(small) >= 0)
+    # beyond it: NaN or a set sign bit, never a finite positive weight
+    big = np.clip(np.rint(8.0 * np.linspace(8.94, 60, 5001) + 55.54), 0, 255).astype(np.int64)
+    assert np.all((big == 0x7F) | (big >= 0x80))
+    edge = np.clip(np.rint(8.0 * np.linspace(8.80, 8.94, 101) + 55.54), 0, 255).astype(np.int64)
+    assert set(edge) <= {0x7E, 0x7F}                          # 448 or NaN: nothing in between is lost silently

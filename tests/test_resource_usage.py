@@ -34,9 +34,8 @@ AUTO_PICKED = {
     "fmha_fwd_kernel16p<256,32,4,1,0,0,0,0,2,0,1,1>": (0, ""),
     "fmha_fwd_kernel<256,32,4,1,0,0,0,0,1,4,0,0>": (0, ""),
     "fmha_fwd_kernel<256,32,4,1,0,0,0,0,1,0,0,0>": (0, ""),
-    # e4m3: big problems at head dim 128 from 4096 keys run the hand-scheduled persistent build (one register spilled once per
-    # workgroup, in front of the item loop)
-    "fmha_fwd_kernel8p<128,64,8,2,1,1,0,0,2,0,0,1>": (1, "outside the loop"),
+    # e4m3: big problems at head dim 128 from 4096 keys run the hand-scheduled persistent build
+    "fmha_fwd_kernel8p<128,64,8,2,1,1,0,0,2,0,0,1>": (0, ""),
     "fmha_fwd_kernel<64,64,4,3,1,1,0,0,1,0,0,0>": (0, ""),
     "fmha_fwd_kernel<128,64,8,2,1,1,0,0,2,0,0,0>": (12, "between the two passes"),
     "fmha_fwd_kernel<128,64,4,2,1,1,0,0,1,0,0,0>": (0, ""),
@@ -79,7 +78,7 @@ def test_auto_picked_kernels_stay_within_their_spill_allowance(kernels):
     k = kernels["fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"]
     assert k["occupancy"] == 2 and k["vgprs"] + k["agprs"] <= 256 and k["scratch"] <= 16
     k = kernels["fmha_fwd_kernel8p<128,64,8,2,1,1,0,0,2,0,0,1>"]
-    assert k["occupancy"] == 2 and k["vgprs"] + k["agprs"] <= 256 and k["scratch"] <= 8
+    assert k["occupancy"] == 2 and k["vgprs"] + k["agprs"] <= 256 and k["scratch"] == 0
 
 
 def test_no_kernel_spills_more_than_the_table_says(kernels):
