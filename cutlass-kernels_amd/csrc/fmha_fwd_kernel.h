@@ -877,17 +877,30 @@ constexpr bool fits(int sq, int skv) {
          (!C::ASM || skv >= (C::QK8 ? 64 : 8) * C::BN);
 }
 
+// Where a hand-scheduled persistent build (one workgroup per CU, each walking its share of the work items) beats the
+// one-workgroup-per-item builds: measured over problem sizes (300 launches each, N(0,1) data).  fp16, all three head
+// dims: from more items than half the CUs on (160 items +30 %, 256 items +21..28 %, 320 items +8 %; at 128 items a tie).
+// e4m3: from 160 items on (+13 %; at 128 items -11 %) and only while the last round of items keeps four fifths of the
+// workgroups busy (320 items -10 %, 384 items -6 %: the 128-row tile has twice the workgroups to even out the tail).
+template <class C>
+constexpr bool hand_loop_pays(long long items) {
+  if (!C::QK8) return items > 128;
+  const long long rounds = (items + 255) / 256;
+  return items >= 160 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
+}
+
 // Calls f with the first instantiation of the list that fits the shape and the wish.  Without a wish for the query
-// rows, tiles above 128 rows and the 16x16x32 builds (slower where launch and prologue dominate) are only taken for
-// big problems (size 2: enough workgroups to fill 256 CUs twice), and the key-split build only for small ones (size 0:
-// its 32-row workgroups fit on the chip all at once).
+// rows, the hand-scheduled builds are taken where they pay (above), other tiles above 128 rows and the other 16x16x32
+// builds (slower where launch and prologue dominate) only for big problems (size 2: enough workgroups to fill 256 CUs
+// twice), and the key-split build only for small ones (size 0: its 32-row workgroups fit on the chip all at once).
 template <class F, class... Cs>
-bool first_fit(CfgList<Cs...>, int sq, int skv, int size, TileWish w, F &&f) {
+bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish w, F &&f) {
   bool done = false;
   auto try_one = [&](auto c) {
     using C = decltype(c);
     if (done || !fits<C>(sq, skv)) return;
-    if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : ((C::BM > 128 || C::M16) && size != 2))) return;
+    const bool by_size = C::ASM ? hand_loop_pays<C>(bh * (sq / C::BM)) : !((C::BM > 128 || C::M16) && size != 2);
+    if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : !by_size)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
     if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;
     if (w.hand && C::ASM != (w.hand > 0)) return;
@@ -906,12 +919,12 @@ void select_tile(int sq, int skv, int bh, F &&f) {
   const bool small = (long long)bh * ((sq + 31) / 32) <= 256 && skv >= 128;
   const int size = big ? 2 : small ? 0 : 1;
   const TileWish w = tile_wish();
-  if ((w.bm || w.bn) && first_fit(All{}, sq, skv, size, w, f)) return;
+  if ((w.bm || w.bn) && first_fit(All{}, sq, skv, bh, size, w, f)) return;
   static const bool no_hand = [] { const char *e = getenv("CFK_FMHA_HANDLOOP"); return e && e[0] == '0'; }();
   // (the hand-scheduled build is a two-pass kernel: not for callers that asked for a data-independent run time)
-  if (first_fit(Auto{}, sq, skv, size, TileWish{0, 0, 0, no_hand || predictable_latency() ? -1 : 0}, f)) return;
+  if (first_fit(Auto{}, sq, skv, bh, size, TileWish{0, 0, 0, no_hand || predictable_latency() ? -1 : 0}, f)) return;
   // query lengths that only the 32-row (key-split) build divides
-  if (first_fit(Auto{}, sq, skv, 0, TileWish{32, 0, 0, 0}, f)) return;
+  if (first_fit(Auto{}, sq, skv, bh, 0, TileWish{32, 0, 0, 0}, f)) return;
   f(Fallback{});
 }
 
