@@ -99,8 +99,8 @@ int cfk_fmha_forward_plan(const cfk_fmha_fwd_params *params, int32_t *block_m, i
                           int32_t *lds_bytes, int32_t *threads);
 
 /* The MFMA shape of the kernel build the library would pick for `params`: 32 (32x32x16 / 32x32x64 MFMAs) or 16
- * (16x16x32; fp16 operands at head dims 64 and 128, big problems -- the more power-efficient shape on this board -- and
- * small ones, whose 32-row workgroups split the keys over their waves).  No
+ * (16x16x32; fp16 operands: problems with more work items than half the CUs -- the more power-efficient shape on this
+ * board -- and small ones at head dims 64 and 128, whose 32-row workgroups split the keys over their waves).  No
  * counterpart in the reference, whose MMA atom is fixed at compile time (src/fmha-pipeline/ss_helper.h:3-94).  The
  * environment variable CFK_FMHA_TILE=<query rows>x<keys>[/16|/16h|/32] overrides the automatic choice of tile and shape
  * (16h / 32h: the builds with the hand-scheduled main loop and persistent workgroups, fp16 / e4m3 at head dim 128; 32x64:
@@ -155,8 +155,8 @@ int cfk_gemm(const cfk_gemm_params *p, void *stream);
 typedef enum cfk_option {
   /* 1: no optimistic first pass.  Two kernels first walk the keys with a softmax reference point fixed by the first key
    * tile (no row max per tile) and, only if some weight left the range of P's type, walk them again tracking the running
-   * max as the reference does on every tile (online_softmax.h:123-165): e4m3 P from 2048 keys on, and fp16 at head dim
-   * 128 on big problems.  On scores that climb along the key axis that costs up to twice the time.  With this option
+   * max as the reference does on every tile (online_softmax.h:123-165): e4m3 P from 4096 keys on, and fp16 problems
+   * with more work items than half the CUs.  On scores that climb along the key axis that costs up to twice the time.  With this option
    * every call takes the max-tracking path from the start: the same results to rounding, a run time that does not
    * depend on the data (a few per cent slower on ordinary data).  0 (default): two passes where they pay. */
   CFK_OPT_PREDICTABLE_LATENCY = 1,
