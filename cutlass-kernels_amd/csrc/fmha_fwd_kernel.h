@@ -878,13 +878,16 @@ constexpr bool fits(int sq, int skv) {
 }
 
 // Where a hand-scheduled persistent build (one workgroup per CU, each walking its share of the work items) beats the
-// one-workgroup-per-item builds: measured over problem sizes (300 launches each, N(0,1) data).  fp16, all three head
-// dims: from more items than half the CUs on (160 items +30 %, 256 items +21..28 %, 320 items +8 %; at 128 items a tie).
+// one-workgroup-per-item builds: measured over problem sizes (driver/run_problem_sizes.sh; 300 launches each, N(0,1)
+// data).  fp16 at head dim 256, where both kinds of build have 128-row items: at every item count from 512 keys on
+// (+25..30 % at 8192 keys, +10..20 % at 1024 and 2048, level at 512; -15 % at 256 keys: eight tiles, all head and tail).  fp16
+// at head dims 64 and 128: from more 256-row items than half the CUs on (160 items +25 %, 256 items +23..28 %, 320 items
+// +9 %; at 128 items a tie, at 96 -4 %: there the 128-row tile's twice as many workgroups count).
 // e4m3: from 160 items on (+13 %; at 128 items -11 %) and only while the last round of items keeps four fifths of the
 // workgroups busy (320 items -10 %, 384 items -6 %: the 128-row tile has twice the workgroups to even out the tail).
 template <class C>
-constexpr bool hand_loop_pays(long long items) {
-  if (!C::QK8) return items > 128;
+constexpr bool hand_loop_pays(long long items, int skv) {
+  if (!C::QK8) return C::BM == 128 ? skv >= 512 : items > 128;
   const long long rounds = (items + 255) / 256;
   return items >= 160 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
 }
@@ -899,7 +902,7 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish
   auto try_one = [&](auto c) {
     using C = decltype(c);
     if (done || !fits<C>(sq, skv)) return;
-    const bool by_size = C::ASM ? hand_loop_pays<C>(bh * (sq / C::BM)) : !((C::BM > 128 || C::M16) && size != 2);
+    const bool by_size = C::ASM ? hand_loop_pays<C>(bh * (sq / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
     if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : !by_size)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
     if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;
