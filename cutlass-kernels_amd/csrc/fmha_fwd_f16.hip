@@ -33,6 +33,8 @@ using N128_128x128 = FmhaCfg<128, 64, 4, 2, false, false, false, false, 2, 0, tr
 // ... and with the hand-scheduled main loop (key length a multiple of 256, at least 512)
 using A128_256x128 = FmhaCfg<128, 64, 8, 2, false, false, false, false, 2, 0, true, true>;
 using A64_256x128 = FmhaCfg<64, 64, 8, 2, false, false, false, false, 2, 0, true, true>;
+using A128_128x128 = FmhaCfg<128, 64, 4, 1, false, false, false, false, 2, 0, true, true>;   // the same loops, 4 waves, one per SIMD
+using A64_128x128 = FmhaCfg<64, 64, 4, 1, false, false, false, false, 2, 0, true, true>;
 
 // ... and for small grids: 32 query rows per workgroup, the eight waves split the keys (fmha_fwd_kernel_ks.h)
 using K64_32x64 = KsCfg<64, 8>;
@@ -43,8 +45,8 @@ using C64Tap = FmhaCfg<64, 64, 4, 2, false, false, false, true>;
 using C128Tap = FmhaCfg<128, 64, 4, 2, false, false, false, true>;
 using C256Tap = FmhaCfg<256, 32, 4, 1, false, false, false, true>;
 
-using All64 = CfgList<C64_128x64, N64_128x64, C64_256x64, C64_128x128, C64_256x128, A64_256x128, K64_32x64>;
-using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128, N128_128x128, A128_256x128, N128_256x128, K128_32x64>;
+using All64 = CfgList<C64_128x64, N64_128x64, C64_256x64, C64_128x128, C64_256x128, A64_256x128, A64_128x128, K64_32x64>;
+using All128 = CfgList<C128_128x64, N128_128x64, C128_256x64P, C128_256x64, N128_256x64, C128_128x128, C128_256x128, N128_128x128, A128_256x128, A128_128x128, N128_256x128, K128_32x64>;
 
 template <class F>
 bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
@@ -57,8 +59,8 @@ bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
     }
   }
   switch (head_dim) {
-    case 64: select_tile<All64, CfgList<K64_32x64, A64_256x128, N64_128x64, C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
-    case 128: select_tile<All128, CfgList<K128_32x64, A128_256x128, N128_256x128, N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
+    case 64: select_tile<All64, CfgList<K64_32x64, A64_256x128, A64_128x128, N64_128x64, C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
+    case 128: select_tile<All128, CfgList<K128_32x64, A128_256x128, A128_128x128, N128_256x128, N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
     default: return false;
   }
 }

@@ -115,7 +115,8 @@ struct FmhaCfg {
   static_assert(SUB == 1 || SUB == 2, "sub-tiles per barrier");
   static_assert(!KPRE || SUB == 1, "K fragment prefetch is a variant of the one-tile step");
   static_assert(!ASM || ((M16 != (QK8 && PV8 && !VT)) && QK8 == PV8 && SUB == 2 &&
-                         ((D == 128 && BN == 64 && NWAVES == 8 && WPE == 2) || (M16 && D == 256 && BN == 32 && NWAVES == 4 && WPE == 1) ||
+                         ((D == 128 && BN == 64 && NWAVES == 8 && WPE == 2) || (M16 && D <= 128 && BN == 64 && NWAVES == 4 && WPE == 1) ||
+                          (M16 && D == 256 && BN == 32 && NWAVES == 4 && WPE == 1) ||
                           (M16 && D == 64 && BN == 64 && NWAVES == 8 && WPE == 2))),
                 "the hand-scheduled loops: fp16 on 16x16x32 MFMAs (head dims 64, 128, 256), e4m3 with V in [B,S,H,D] (128)");
   static_assert(BN % 32 == 0 && (!PV8 || BN == 64), "key tile: the e4m3 second GEMM has 64-deep K-steps");
@@ -882,12 +883,14 @@ constexpr bool fits(int sq, int skv) {
 // data).  fp16 at head dim 256, where both kinds of build have 128-row items: at every item count from 512 keys on
 // (+25..30 % at 8192 keys, +10..20 % at 1024 and 2048, level at 512; -15 % at 256 keys: eight tiles, all head and tail).  fp16
 // at head dims 64 and 128: from more 256-row items than half the CUs on (160 items +25 %, 256 items +23..28 %, 320 items
-// +9 %; at 128 items a tie, at 96 -4 %: there the 128-row tile's twice as many workgroups count).
+// +9 %; at 128 items a tie, at 96 -4 %: there the 128-row tile's twice as many workgroups count).  Up to 256 items of 128
+// rows -- one round -- those head dims take the same loops in their 4-wave shape (128 rows, one wave per SIMD): +11..20 %
+// over the compiler-scheduled 128-row builds from 1024 keys on (2048 keys +12 %, 8192 +20 %, 1024 +2..6 %, 512 -5 %).
 // e4m3: from 160 items on (+13 %; at 128 items -11 %) and only while the last round of items keeps four fifths of the
 // workgroups busy (320 items -10 %, 384 items -6 %: the 128-row tile has twice the workgroups to even out the tail).
 template <class C>
 constexpr bool hand_loop_pays(long long items, int skv) {
-  if (!C::QK8) return C::BM == 128 ? skv >= 512 : items > 128;
+  if (!C::QK8) return C::D == 256 ? skv >= 512 : C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;
   const long long rounds = (items + 255) / 256;
   return items >= 160 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
 }

@@ -2,6 +2,8 @@
 """Generator of the hand-scheduled main loops of the fp16 FMHA forward kernel on 16x16x32 MFMAs (fmha_fwd_kernel16p.h,
 FmhaCfg::ASM), in three shapes:
   d128  head dim 128, 64-key tiles, 256 query rows per workgroup (8 waves x 32 rows, two waves per SIMD)
+  d128w4, d64w4  the d128 / d64 loops for 128 query rows per workgroup: 4 waves, one per SIMD, O in the accumulation
+        registers (for problems with too few 256-row work items to go round)
   d64   head dim 64, 64-key tiles of 8 KB, 256 query rows per workgroup (8 waves, two per SIMD); 36 MFMA slots per tile:
         here the softmax (112 vector instructions beside 32 MFMAs) is what fills the issue port, so the row sum goes to
         the matrix pipe (ROWSUM = "mfma")
@@ -9,7 +11,7 @@ FmhaCfg::ASM), in three shapes:
         are 192 registers per lane; O lives in the accumulation registers a[0:127])
 d128 and d256 have the same timeline (64 MFMA slots and 16 KB of K and of V per tile); the text below describes d128.
 
-    python3 gen_fmha_loop16.py            # rewrites fmha_fwd_loop16_{d128,d256,d64}.inc beside this file
+    python3 gen_fmha_loop16.py            # rewrites fmha_fwd_loop16_{d128,d128w4,d256,d64,d64w4}.inc beside this file
     python3 gen_fmha_loop16.py --check    # exit status 1 if those files are not what the generator produces
 
 Why a generator: the loop is one inline-asm statement of ~2800 instructions with every register assigned by hand.
@@ -91,9 +93,15 @@ def configure():
     g = globals()
     if SHAPE == "d128":
         g.update(D=128, BN=64, NWAVES=8, O_ACC=False, O0=192, SA0=128, SB0=160, Q0=96, P0=80, RING0=48, KRD0=24, VRD0=28, GOK0=36, GOV0=38)
+    elif SHAPE == "d128w4":   # the same loop for 128 query rows: 4 waves, one per SIMD, four copies per wave and tile, O in a[0:63]
+        assert ROWSUM == "add" and FOLD
+        g.update(D=128, BN=64, NWAVES=4, O_ACC=True, O0=0, SA0=128, SB0=160, Q0=96, P0=80, RING0=48, KRD0=24, VRD0=28, GOK0=192, GOV0=196)
     elif SHAPE == "d64":
         assert ROWSUM == "mfma"
         g.update(D=64, BN=64, NWAVES=8, O_ACC=False, O0=224, SA0=160, SB0=192, Q0=144, P0=128, RING0=96, KRD0=82, VRD0=78, GOK0=77, GOV0=76)
+    elif SHAPE == "d64w4":    # ... and the head-dim-64 loop for 128 query rows: 4 waves, two copies per wave and tile, O in a[0:31]
+        assert ROWSUM == "mfma" and FOLD
+        g.update(D=64, BN=64, NWAVES=4, O_ACC=True, O0=0, SA0=160, SB0=192, Q0=144, P0=128, RING0=96, KRD0=82, VRD0=78, GOK0=224, GOV0=226)
     else:
         assert ROWSUM == "add"
         g.update(D=256, BN=32, NWAVES=4, O_ACC=True, O0=0, SA0=224, SB0=240, Q0=160, P0=144, RING0=112, KRD0=96, VRD0=80, GOK0=72, GOV0=76)
@@ -105,7 +113,7 @@ def configure():
     if SHAPE == "d256":
         g.update(M0R=70, MN0=104, LA0=64, QOFF0=68, LOW=64, L_OUT=(64, 66), T=64, L_TOTAL=False)
         start = 36   # S(t+1) is complete at slot 32; P(t+1) has to be before slot 32 of the next period
-    elif SHAPE == "d64":
+    elif SHAPE in ("d64", "d64w4"):
         g.update(M0R=74, MN0=64, ONES0=92, LACC0=84, QOFF0=72, LOW=64 if FOLDED else 72, L_OUT=(84, 88), T=36, L_TOTAL=True)
         start = 23   # P(t)'s first half is consumed by slot 26; P(t+1)'s second half is needed at slot 26 of the next period
     elif ROWSUM == "mfma" and FOLDED:
@@ -114,7 +122,7 @@ def configure():
     elif ROWSUM == "mfma":
         g.update(M0R=18, ONES0=20, LACC0=40, QOFF0=16, LOW=16, L_OUT=(40, 44), T=68, L_TOTAL=True)
         start = 46
-    elif ROWSUM == "add" and FOLDED:
+    elif ROWSUM == "add" and FOLDED:   # (d128 and d128w4)
         g.update(MN0=40, LA0=18, QOFF0=22, LOW=18, L_OUT=(18, 20), T=64, L_TOTAL=False)
         start = 44
     elif ROWSUM == "add":
@@ -411,7 +419,13 @@ def render():
     used |= set(range(GOK0, GOK0 + IPW)) | set(range(GOV0, GOV0 + IPW)) | {QOFF0, QOFF0 + 1} | set(L_OUT)
     used |= {MN0, MN0 + 4} if FOLDED else {M0R, M0R + 1}
     if not O_ACC: used |= set(range(O0, O0 + 16 * n_o))
-    clob = ['"memory"', '"scc"', '"m0"'] + ['"v%d"' % r for r in range(LOW, 256) if r not in used]
+    # (vector registers the loop never names stay the compiler's: values it keeps across the statement need not be spilled)
+    import re
+    named = set()
+    for ins in head + body + tail:
+        for m in re.finditer(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b", ins):
+            named |= set(range(int(m.group(1)), int(m.group(2)) + 1)) if m.group(1) else {int(m.group(3))}
+    clob = ['"memory"', '"scc"', '"m0"'] + ['"v%d"' % r for r in range(LOW, 256) if r not in used and r in named]
     L.append("    : " + ", ".join(clob) + ");")
     return "\n".join(L) + "\n"
 
@@ -421,7 +435,7 @@ if __name__ == "__main__":
     overrides = json.loads(os.environ.get("LOOP16_SET", "{}"))
     stale = False
     defaults = {k: globals()[k] for k in overrides}
-    for shape, rowsum in (("d128", "add"), ("d256", "add"), ("d64", "mfma")):
+    for shape, rowsum in (("d128", "add"), ("d128w4", "add"), ("d256", "add"), ("d64", "mfma"), ("d64w4", "mfma")):
         SHAPE, ROWSUM = shape, rowsum
         for k, v in overrides.items():
             if isinstance(v, dict): v = v.get(shape, rowsum if k == "ROWSUM" else defaults[k])   # {"ROWSUM": {"d128": "mfma"}}: one shape only

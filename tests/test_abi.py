@@ -149,7 +149,10 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     # where the hand-scheduled persistent builds start (one workgroup per CU): fp16 from more 256-row items than half the
     # CUs (head dim 256, 128-row items on either side: always); e4m3 from 160 items, while the last round keeps four
     # fifths of the CUs busy
-    assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 1, 16, 2048, 2048, 128)        # 128 items
+    assert f.fmha_forward_kernel(f.CFK_FP16, 1, 16, 2048, 2048, 128) == "fmha_fwd_kernel16p<128,64,4,1,0,0,0,0,2,0,1,1>"   # 128 items: the 4-wave shape
+    assert f.fmha_forward_kernel(f.CFK_FP16, 1, 6, 2048, 2048, 64) == "fmha_fwd_kernel16p<64,64,4,1,0,0,0,0,2,0,1,1>"     # (up to 256 items of 128 rows,
+    assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 1, 64, 512, 512, 128)                                    #  from 1024 keys)
+    assert f.fmha_forward_kernel(f.CFK_FP16, 1, 2, 2048, 2048, 128) == "fmha_fwd_kernel_ks<128,8>"                        # small grids: the key-split build
     assert "kernel16p<128" in f.fmha_forward_kernel(f.CFK_FP16, 1, 20, 2048, 2048, 128)         # 160
     assert "kernel16p<128" in f.fmha_forward_kernel(f.CFK_FP16, 1, 40, 2048, 2048, 128)         # 320
     assert "kernel16p<64" in f.fmha_forward_kernel(f.CFK_FP16, 1, 24, 2048, 2048, 64)

@@ -1,6 +1,8 @@
 """Symbolic check of the hand-scheduled main loops of the fp16 kernel (cutlass-kernels_amd/csrc/gen_fmha_loop16.py), in
-its three shapes (head dim 128: 8 waves, 64-key tiles; head dim 256: 4 waves, 32-key tiles, O in accumulation registers;
-head dim 64: 8 waves, 64-key tiles of 8 KB, row sum on the matrix pipe).
+its five shapes (head dim 128: 8 waves, 64-key tiles; head dim
+256: 4 waves, 32-key tiles, O in accumulation registers;
+head dim 64: 8 waves, 64-key tiles of 8 KB, row sum on the matrix pipe; head dims 128 and 64 again for 4 waves with O
+in accumulation registers).
 
 A loop is ~2800 hand-allocated instructions inside one asm statement, where neither the compiler's register
 allocator nor its hazard recognizer helps.  This test walks the instruction text a wave executes (loop unrolled for
@@ -354,8 +356,8 @@ class Checker:
         assert self.idx - last_mfma > 8
 
 
-@pytest.mark.parametrize("shape,rowsum,fold", [("d128", "mfma", False), ("d128", "mfma", True), ("d128", "add", True), ("d128", "add", False), ("d128", "dot", False),
-                                               ("d256", "add", True), ("d256", "add", False), ("d64", "mfma", True), ("d64", "mfma", False)])
+@pytest.mark.parametrize("shape,rowsum,fold", [("d128", "mfma", False), ("d128", "mfma", True), ("d128", "add", True), ("d128w4", "add", True), ("d128", "add", False), ("d128", "dot", False),
+                                               ("d256", "add", True), ("d256", "add", False), ("d64", "mfma", True), ("d64", "mfma", False), ("d64w4", "mfma", True)])
 @pytest.mark.parametrize("n_tiles", [8, 12, 16, 32, 64])
 def test_loop_is_correct_symbolically(n_tiles, shape, rowsum, fold):
     g = _gen()
@@ -367,10 +369,10 @@ def test_loop_is_correct_symbolically(n_tiles, shape, rowsum, fold):
     c.finish()
 
 
-@pytest.mark.parametrize("shape", ["d128", "d256", "d64"])
+@pytest.mark.parametrize("shape", ["d128", "d128w4", "d256", "d64", "d64w4"])
 def test_checker_catches_a_broken_schedule(shape):
     g = _gen()
-    g.SHAPE, g.ROWSUM = shape, ("mfma" if shape == "d64" else "add")
+    g.SHAPE, g.ROWSUM = shape, ("mfma" if shape.startswith("d64") else "add")
     g.configure()
     prog = g.program(8)
     # drop one LDS wait: some MFMA then reads a fragment that was not waited for
@@ -392,4 +394,4 @@ def test_checker_catches_a_broken_schedule(shape):
 
 def test_committed_include_is_the_generators_output():
     r = subprocess.run([sys.executable, os.path.join(CSRC, "gen_fmha_loop16.py"), "--check"])
-    assert r.returncode == 0, "fmha_fwd_loop16_{d128,d256,d64}.inc are stale: run gen_fmha_loop16.py"
+    assert r.returncode == 0, "fmha_fwd_loop16_{d128,d128w4,d256,d64,d64w4}.inc are stale: run gen_fmha_loop16.py"

@@ -26,6 +26,9 @@ AUTO_PICKED = {
     # fp16, small grids (the waves split the keys)
     "fmha_fwd_kernel_ks<64,8>": (0, ""),
     "fmha_fwd_kernel_ks<128,8>": (0, ""),
+    # ... and its 4-wave shapes (128 query rows, one wave per SIMD) for up to 256 items of 128 rows
+    "fmha_fwd_kernel16p<128,64,4,1,0,0,0,0,2,0,1,1>": (0, ""),
+    "fmha_fwd_kernel16p<64,64,4,1,0,0,0,0,2,0,1,1>": (0, ""),
     # fp16 head dim 64: big problems run the hand-scheduled persistent build
     "fmha_fwd_kernel16p<64,64,8,2,0,0,0,0,2,0,1,1>": (0, ""),
     "fmha_fwd_kernel16<64,64,4,3,0,0,0,0,1,0,1,0>": (14, "the slow path of the row-sum test"),

@@ -40,6 +40,13 @@ CASES = {
     # 3x6 heads x 2048 rows = 288 items of 128 rows (32 workgroups take a second one), climbing keys, taps
     "128x64/16h": ["f16nt:1,256,2,256", "f16nt:1,128,3,256,640", "f16nt:3,2048,6,256,512", "f16ntclimb:1,256,2,256,512",
                    "f16ntclimb:3,1024,12,256,256", "f16:1,256,2,256,384", "f16climb:1,256,2,256,512"],
+    # ... and the head-dim-128 loop for 128 query rows (4 waves, one per SIMD, O in accumulation registers): 1x20 heads x
+    # 2048 rows = 320 items (64 workgroups take a second one), climbing keys, taps
+    "128x128/16h": ["f16nt:1,256,2,128,512", "f16nt:1,128,3,128,768", "f16nt:1,2048,20,128", "f16nt:2,384,3,128,1024", "f16ntclimb:1,256,2,128,768",
+                    "f16ntclimb:5,1024,8,128", "f16:1,256,2,128,512", "f16climb:1,256,2,128,768",
+                    # ... and the head-dim-64 loop likewise
+                    "f16nt:1,256,2,64,512", "f16nt:1,128,3,64,768", "f16nt:1,2048,20,64", "f16ntclimb:1,256,2,64,768", "f16ntclimb:5,1024,8,64",
+                    "f16:1,256,2,64,512", "f16climb:1,256,2,64,1024"],
     # the e4m3 build with the hand-scheduled loop and persistent workgroups (key length a multiple of 256, from 4096): the
     # scheduled loop, 4352 keys (an odd number of loop turns), 2x10 heads x 4096 rows = 320 items (a quarter of the
     # workgroups take a second one), climbing keys (the vote, the max-tracking loop, then a next item: 5x13x1024 rows = 260)
