@@ -880,8 +880,9 @@ constexpr bool fits(int sq, int skv) {
 
 // Where a hand-scheduled persistent build (one workgroup per CU, each walking its share of the work items) beats the
 // one-workgroup-per-item builds: measured over problem sizes (driver/run_problem_sizes.sh; 300 launches each, N(0,1)
-// data).  fp16 at head dim 256, where both kinds of build have 128-row items: at every item count from 512 keys on
-// (+25..30 % at 8192 keys, +10..20 % at 1024 and 2048, level at 512; -15 % at 256 keys: eight tiles, all head and tail).  fp16
+// data).  fp16 at head dim 256, where both kinds of build have 128-row items: at every item count from 1024 keys on
+// (+25..30 % at 8192 keys, +10..20 % at 1024 and 2048; -1..-4 % at 512, -15 % at 256 keys: eight tiles, all head and
+// tail).  fp16
 // at head dims 64 and 128: from more 256-row items than half the CUs on (160 items +25 %, 256 items +23..28 %, 320 items
 // +9 %; at 128 items a tie, at 96 -4 %: there the 128-row tile's twice as many workgroups count).  Up to 256 items of 128
 // rows -- one round -- those head dims take the same loops in their 4-wave shape (128 rows, one wave per SIMD): +11..20 %
@@ -890,7 +891,7 @@ constexpr bool fits(int sq, int skv) {
 // workgroups busy (320 items -10 %, 384 items -6 %: the 128-row tile has twice the workgroups to even out the tail).
 template <class C>
 constexpr bool hand_loop_pays(long long items, int skv) {
-  if (!C::QK8) return C::D == 256 ? skv >= 512 : C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;
+  if (!C::QK8) return C::D == 256 ? skv >= 1024 : C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;
   const long long rounds = (items + 255) / 256;
   return items >= 160 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
 }

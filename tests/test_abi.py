@@ -157,9 +157,9 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     assert "kernel16p<128" in f.fmha_forward_kernel(f.CFK_FP16, 1, 40, 2048, 2048, 128)         # 320
     assert "kernel16p<64" in f.fmha_forward_kernel(f.CFK_FP16, 1, 24, 2048, 2048, 64)
     assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 3, 8192, 8192, 256)          # 192 items of 128 rows
-    assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 1, 8192, 8192, 256)          # (at head dim 256 from 512 keys)
-    assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 2, 512, 512, 256)
-    assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 16, 64, 256, 256, 256)
+    assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 1, 8192, 8192, 256)          # (at head dim 256 from 1024 keys)
+    assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 2, 1024, 1024, 256)
+    assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 16, 64, 512, 512, 256)
     assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 1, 40, 2048, 2048 + 64, 128)   # key length: whole 256s only
     assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 8, 4096, 4096, 128)      # 128 items
     assert "kernel8p<" in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 10, 4096, 4096, 128)         # 160

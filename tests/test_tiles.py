@@ -73,13 +73,11 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
         return subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout.strip()
     # medium problems: 128-row tiles; small ones (the last: 128 workgroups of 32 rows fit on the chip at once): fp16 at head
     # dims 64 and 128 takes 32-row workgroups whose waves split the keys
-    # (head dim 256 with 512 keys: the hand-scheduled 128 x 64 build, whatever the wish -- none of the wished tiles exists there)
-    assert plans(None) == "(128, 64) (128, 64) (128, 64) (128, 64) (32, 64)"
-    assert plans("256x128") == "(256, 128) (128, 64) (256, 128) (128, 64) (256, 128)"     # no such tile at head dim 256; 384 % 256 != 0
-    assert plans("large") == "(256, 64) (128, 64) (256, 64) (128, 64) (256, 64)"
-    assert plans("128x128") == "(128, 128) (128, 64) (128, 128) (128, 128) (128, 128)"
-    assert plans("32x64") == "(32, 64) (128, 64) (128, 64) (32, 64) (32, 64)"              # fp16 at head dims 64 / 128 only
-    assert plans("128x32") == "(128, 64) (128, 32) (128, 64) (128, 64) (32, 64)"           # head dim 256 only: the compiler-scheduled tile
+    assert plans(None) == "(128, 64) (128, 32) (128, 64) (128, 64) (32, 64)"
+    assert plans("256x128") == "(256, 128) (128, 32) (256, 128) (128, 64) (256, 128)"     # no such tile at head dim 256; 384 % 256 != 0
+    assert plans("large") == "(256, 64) (128, 32) (256, 64) (128, 64) (256, 64)"
+    assert plans("128x128") == "(128, 128) (128, 32) (128, 128) (128, 128) (128, 128)"
+    assert plans("32x64") == "(32, 64) (128, 32) (128, 64) (32, 64) (32, 64)"              # fp16 at head dims 64 / 128 only
     # the MFMA shape suffix: served for fp16 at head dims 64/128 only (e4m3 and head dim 256 ignore the wish)
     mfma_code = ("import sys; sys.path.insert(0, %r); import __graft_entry__ as e; p = e.load_package(); f = p.fmha; "
                  "print(f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 128), f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 64), "
@@ -88,15 +86,13 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     def shapes(wish):
         env = dict(os.environ, CFK_FMHA_TILE=wish)
         return subprocess.run([sys.executable, "-c", mfma_code], env=env, capture_output=True, text=True, check=True).stdout.strip()
-    # (third figure: head dim 256, where none of these wishes but 128x64 names a built tile -- the automatic choice
-    # there is the hand-scheduled build on 16x16x32 MFMAs)
-    assert shapes("128x64/16") == "16 16 16 32 (128, 64)"
-    assert shapes("256x64/16") == "16 32 16 32 (256, 64)"      # no 256-row 16x16x32 build at head dim 64
-    assert shapes("256x64/32") == "32 32 16 32 (256, 64)"
+    assert shapes("128x64/16") == "16 16 32 32 (128, 64)"
+    assert shapes("256x64/16") == "16 32 32 32 (256, 64)"      # no 256-row 16x16x32 build at head dim 64
+    assert shapes("256x64/32") == "32 32 32 32 (256, 64)"
     assert shapes("128x64") == "32 32 32 32 (128, 64)"
-    assert shapes("256x128") == "32 32 16 32 (256, 128)"
-    assert shapes("256x128/16") == "16 32 16 32 (256, 128)"   # two key tiles per barrier on 16x16x32: head dim 128 only
-    assert shapes("256x128/16h") == "16 16 16 32 (256, 128)"  # ... with the hand-scheduled loop: head dims 128 and 64
+    assert shapes("256x128") == "32 32 32 32 (256, 128)"
+    assert shapes("256x128/16") == "16 32 32 32 (256, 128)"   # two key tiles per barrier on 16x16x32: head dim 128 only
+    assert shapes("256x128/16h") == "16 16 32 32 (256, 128)"  # ... with the hand-scheduled loop: head dims 128 and 64
     # the hand-scheduled build needs 160 KB of LDS; a wish for the compiler-scheduled one (no `h`) is kept apart from it
     lds_code = ("import sys; sys.path.insert(0, %r); import __graft_entry__ as e; p = e.load_package(); f = p.fmha; "
                 "print(f.fmha_forward_plan(f.CFK_FP16, 2, 4, 1536, 512, 128)[2], f.fmha_forward_plan(f.CFK_FP16, 2, 4, 1536, 384, 128)[:3])" % ROOT)
@@ -120,8 +116,8 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     assert f.fmha_forward_mfma(f.CFK_FP16, 2, 8, 8192, 8192, 256) == 16                             # hand-scheduled, 16x16x32
     assert f.fmha_forward_kernel(f.CFK_FP16, 2, 8, 8192, 8192, 256) == "fmha_fwd_kernel16p<256,32,4,1,0,0,0,0,2,0,1,1>"
     assert f.fmha_forward_kernel(f.CFK_FP16, 2, 8, 8192, 8160, 256) == "fmha_fwd_kernel<256,32,4,1,0,0,0,0,1,0,0,0>"   # key length % 128 != 0
-    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 256) == 16                              # ... from 512 keys on
-    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 256, 256) == 32                              # below: 32x32
+    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 1024, 256) == 16                             # ... from 1024 keys on
+    assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 256) == 32                              # below: 32x32
     assert f.fmha_forward_mfma(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128) == 32
     assert f.fmha_forward_plan(f.CFK_FP8_E4M3, 4, 16, 4096, 4096, 128)[:2] == (256, 128)
 
