@@ -17,6 +17,7 @@ using C128_256x128 = FmhaCfg<128, 64, 8, 2, true, true, false, false, 2>;
 // ... with the hand-scheduled main loop and persistent workgroups (fmha_fwd_kernel8p.h); key sequences from 4096: below,
 // e4m3 weights run the max-tracking pass only (cfk_api.hip), which this build would do in a loop that is not pipelined
 using A128_256x128 = FmhaCfg<128, 64, 8, 2, true, true, false, false, 2, 0, false, true>;
+using A128_128x128 = FmhaCfg<128, 64, 4, 2, true, true, false, false, 2, 0, false, true>;   // the same loop, 4 waves, one per SIMD
 using C256_128x64 = FmhaCfg<256, 64, 4, 1, true, true>;
 using C256_128x128 = FmhaCfg<256, 64, 4, 1, true, true, false, false, 2>;
 
@@ -34,7 +35,7 @@ using C128TTap = FmhaCfg<128, 64, 4, 2, true, true, true, true>;
 using C256TTap = FmhaCfg<256, 64, 4, 1, true, true, true, true>;
 
 using All64 = CfgList<C64_128x64, C64_128x128>;
-using All128 = CfgList<C128_128x64, C128_256x64, C128_128x128, C128_256x128, A128_256x128>;
+using All128 = CfgList<C128_128x64, C128_256x64, C128_128x128, C128_256x128, A128_256x128, A128_128x128>;
 using All256 = CfgList<C256_128x64, C256_128x128>;
 
 template <class F>
@@ -59,7 +60,7 @@ bool dispatch(int head_dim, int sq, int skv, int bh, int v_layout, bool tap_s, F
   switch (head_dim) {
     case 64: select_tile<All64, CfgList<C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
     // big problems: 256 rows with one barrier per 128 keys (+4 % on N(0,1) data over the 128x64 tile)
-    case 128: select_tile<All128, CfgList<A128_256x128, C128_256x128, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
+    case 128: select_tile<All128, CfgList<A128_256x128, A128_128x128, C128_256x128, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
     // one barrier per 128 keys: +11 % at head dim 256 (1604 against 1439 TFLOP/s, B=4 H=8 S=4096)
     case 256: select_tile<All256, CfgList<C256_128x128, C256_128x64>, C256_128x64>(sq, skv, bh, f); return true;
     default: return false;

@@ -116,6 +116,7 @@ struct FmhaCfg {
   static_assert(!KPRE || SUB == 1, "K fragment prefetch is a variant of the one-tile step");
   static_assert(!ASM || ((M16 != (QK8 && PV8 && !VT)) && QK8 == PV8 && SUB == 2 &&
                          ((D == 128 && BN == 64 && NWAVES == 8 && WPE == 2) || (M16 && D <= 128 && BN == 64 && NWAVES == 4 && WPE == 1) ||
+                          (QK8 && D == 128 && BN == 64 && NWAVES == 4 && WPE == 2) ||
                           (M16 && D == 256 && BN == 32 && NWAVES == 4 && WPE == 1) ||
                           (M16 && D == 64 && BN == 64 && NWAVES == 8 && WPE == 2))),
                 "the hand-scheduled loops: fp16 on 16x16x32 MFMAs (head dims 64, 128, 256), e4m3 with V in [B,S,H,D] (128)");
@@ -892,6 +893,7 @@ constexpr bool fits(int sq, int skv) {
 template <class C>
 constexpr bool hand_loop_pays(long long items, int skv) {
   if (!C::QK8) return C::D == 256 ? skv >= 1024 : C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;
+  if (C::BM == 128) return items <= 256;   // (the 4-wave shape: one round of 128-row items)
   const long long rounds = (items + 255) / 256;
   return items >= 160 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
 }

@@ -1,8 +1,9 @@
 #!/usr/bin/env python3
 """Generator of the hand-scheduled main loop of the e4m3 FMHA forward kernel (fmha_fwd_kernel8p.h): head dim 128, 256
-query rows per workgroup (8 waves x 32 rows, two waves per SIMD), 64-key tiles, V in [B,S,H,D].
+query rows per workgroup (8 waves x 32 rows, two waves per SIMD), 64-key tiles, V in [B,S,H,D]; and the same loop for
+128 query rows (NWAVES = 4, one wave per SIMD, two copies per wave and tile: problems with too few 256-row work items).
 
-    python3 gen_fmha_loop8.py            # rewrites fmha_fwd_loop8_d128.inc and fmha_fwd_loop8_d128_direct.inc beside this file
+    python3 gen_fmha_loop8.py            # rewrites fmha_fwd_loop8_d128{,w4}{,_direct}.inc beside this file
     python3 gen_fmha_loop8.py --check    # exit status 1 if those files are not what the generator produces
 
 Why: this kernel is bound by instruction issue, not by the matrix pipe.  Measured with register-only loops (two waves per
@@ -47,7 +48,8 @@ import json
 import os
 import sys
 
-D, BN, NWAVES = 128, 64, 8
+D, BN = 128, 64
+NWAVES = 8                               # 8: 256 query rows, two waves per SIMD; 4: 128 query rows, one wave per SIMD (two copies per wave and tile)
 KB, KS, DB = BN // 32, D // 64, D // 32
 K_PITCH = V_PITCH = D
 K_TILE = V_TILE = BN * K_PITCH          # 8192
@@ -56,7 +58,8 @@ K_ST0, V_ST0 = 0, NSLOT * K_TILE        # LDS map: K slots, then V slots (the re
 T = 9                                    # MFMA places per tile
 
 O0, SA0, SB0, Q0, P0, RING0 = 192, 128, 160, 112, 96, 48
-LACC0, ONES0, KRD0, VRD0, GOK, GOV, MREF, QOFF = 44, 36, 24, 28, 32, 33, 34, 35
+LACC0, ONES0, KRD0, VRD0, MREF, QOFF = 44, 36, 24, 28, 34, 35
+GOK, GOV = (32, 82), (33, 83)            # lane offsets of the wave's K / V copies (the second ones: 4 waves only)
 FLAGS = 80         # DIRECT: OR of all P registers of the item (a byte with bit 7 set is a weight beyond the e4m3 range)
 LOW = 24
 RING = 4
@@ -129,12 +132,18 @@ def softmax_ops(t):
     return ops
 
 
+def ipw(): return K_TILE // 1024 // NWAVES   # copies per wave and tile (K and V alike)
+
+
 def copy_ops(kind, ring_slot):
-    """the wave's global->LDS copy of its eighth of one tile into ring slot `ring_slot`, then the pointer moves on one tile"""
+    """the wave's global->LDS copies of its share of one tile into ring slot `ring_slot` (1 KB each, NWAVES KB apart), then
+    the pointer moves on one tile"""
     base = (K_ST0 if kind == 'K' else V_ST0) + ring_slot * K_TILE
     go, sp = (GOK, 40) if kind == 'K' else (GOV, 42)
-    return [["s_add_u32 m0, %%[ldsw], %d" % base, "s_nop 0", "global_load_lds_dwordx4 v%d, s[%d:%d]" % (go, sp, sp + 1),
-             "s_add_u32 s%d, s%d, %%[stride]" % (sp, sp), "s_addc_u32 s%d, s%d, 0" % (sp + 1, sp + 1)]]
+    ops = [["s_add_u32 m0, %%[ldsw], %d" % (base + i * NWAVES * 1024), "s_nop 0", "global_load_lds_dwordx4 v%d, s[%d:%d]" % (go[i], sp, sp + 1)]
+           for i in range(ipw())]
+    ops[-1] += ["s_add_u32 s%d, s%d, %%[stride]" % (sp, sp), "s_addc_u32 s%d, s%d, 0" % (sp + 1, sp + 1)]
+    return ops
 
 
 def schedule(n_tiles):
@@ -172,7 +181,7 @@ def schedule(n_tiles):
         groups = []
         for kind, t in (('K', 2 * J + 3), ('K', 2 * J + 4), ('V', 2 * J + 2), ('V', 2 * J + 3)):
             if t < n_tiles: groups += copy_ops(kind, t % NSLOT)
-        for i, grp in enumerate(groups): copies_at[SS * J + 1 + 4 * i] = grp
+        for i, grp in enumerate(groups): copies_at[SS * J + 1 + (4 // ipw()) * i] = grp
     # ---- the workgroup's next work item (persistent workgroups): in the last super-step, whose K slots 0-2 and V slots
     # 0-1 are free, copy that item's first three K and two V tiles into them and, once the last S = K.Q^T has been
     # issued, load its Q into the Q registers; both are waited for at the end of the statement
@@ -180,7 +189,7 @@ def schedule(n_tiles):
     copies_at[Z] = ["s_mov_b64 s[40:41], %[kn]", "s_mov_b64 s[42:43], %[vn]"]
     groups = []
     for kind, ring_slot in (('K', 0), ('K', 1), ('K', 2), ('V', 0), ('V', 1)): groups += copy_ops(kind, ring_slot)
-    for i, grp in enumerate(groups): copies_at[Z + 1 + 3 * i] = grp
+    for i, grp in enumerate(groups): copies_at[Z + 1 + (3 * i if ipw() == 1 else i)] = grp
     for i in range(2 * KS):
         copies_at.setdefault(Z + 5 + i, []).append("global_load_dwordx4 %s, v%d, %%[qn] offset:%d" % (vr(q_reg(i // 2) + 4 * (i % 2), 4), QOFF, 64 * (i // 2) + 16 * (i % 2)))
     # ---- emission
@@ -270,12 +279,12 @@ def render():
     sa1 (in, clobbered: S(0) of key blocks 0, 1), qv (in: this item's Q; out: the next item's); f32x4 lacc (out: the row
     sum, complete in every lane); int8v ones (the 0/1 operand); uint64_t kptr, vptr (in: this item's K tile 3 / V tile
     2; out: the same of the next item), kn, vn, qn (the next item's K, V and this wave's Q rows); uint32_t nloop,
-    k_rd[4], v_rd[4], goff_k, goff_v, qoff, lds_wave, tile_stride; float m_loop, c_loop; with DIRECT also uint32_t p_flags
+    k_rd[4], v_rd[4], goff_k[], goff_v[] (one per copy of the wave and tile), qoff, lds_wave, tile_stride; float m_loop, c_loop; with DIRECT also uint32_t p_flags
     (out) and constexpr bool kDirect."""
     head, body, tail = folded()
     L = []
     L.append("// GENERATED by gen_fmha_loop8.py -- do not edit.  The hand-scheduled main loop of fmha_fwd_kernel8p (e4m3, head dim")
-    L.append("// 128, 256 x 128): %d + %d (loop) + %d instructions." % (len(head), len(body), len(tail)))
+    L.append("// 128, %d x 128): %d + %d (loop) + %d instructions." % (32 * NWAVES, len(head), len(body), len(tail)))
     L.append("// The weights are built as e4m3 codes without an exponential: c_loop = 8 c, m_loop = 8 m - 55.54, p_flags = OR of all P (true);")
     L.append("// or with v_exp_f32 and v_cvt_pk_fp8_f32: c_loop = c, m_loop = m (false)")
     L.append("static_assert(kDirect == %s, \"the caller passes the scale and the reference point in the form this loop takes\");" % ("true" if DIRECT else "false"))
@@ -295,11 +304,13 @@ def render():
     L.append('      "+{v[128:143]}"(sa0), "+{v[144:159]}"(sa1), "+{v[112:127]}"(qv), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), [nloop] "+s"(nloop)')
     ins = ['"{v[36:43]}"(ones)', '"{v%d}"(qoff)' % QOFF, '[kn] "s"(kn)', '[vn] "s"(vn)', '[qn] "s"(qn)']
     ins += ['"{v%d}"(k_rd[%d])' % (KRD0 + i, i) for i in range(4)] + ['"{v%d}"(v_rd[%d])' % (VRD0 + i, i) for i in range(DB)]
-    ins += ['"{v%d}"(goff_k)' % GOK, '"{v%d}"(goff_v)' % GOV, '"{v%d}"(m_loop)' % MREF]
+    ins += ['"{v%d}"(goff_k[%d])' % (GOK[i], i) for i in range(ipw())] + ['"{v%d}"(goff_v[%d])' % (GOV[i], i) for i in range(ipw())]
+    ins += ['"{v%d}"(m_loop)' % MREF]
     ins += ['[c] "s"(c_loop)', '[ldsw] "s"(lds_wave)', '[stride] "s"(tile_stride)']
     L.append("    : " + ", ".join(ins))
     used = set(range(O0, O0 + 64)) | set(range(SA0, SA0 + 32)) | set(range(Q0, Q0 + 16)) | set(range(LOW, LACC0 + 4))
     if DIRECT: used.add(FLAGS)
+    used |= set(GOK[:ipw()]) | set(GOV[:ipw()])
     # (registers the loop never names stay the compiler's: values it keeps across the statement need not be spilled)
     import re
     named = set()
@@ -314,7 +325,8 @@ def render():
 if __name__ == "__main__":
     for k, v in json.loads(os.environ.get("LOOP8_SET", "{}")).items(): globals()[k] = v
     stale = False
-    for DIRECT, name in ((False, "fmha_fwd_loop8_d128.inc"), (True, "fmha_fwd_loop8_d128_direct.inc")):
+    for NWAVES, DIRECT, name in ((8, False, "fmha_fwd_loop8_d128.inc"), (8, True, "fmha_fwd_loop8_d128_direct.inc"),
+                                 (4, False, "fmha_fwd_loop8_d128w4.inc"), (4, True, "fmha_fwd_loop8_d128w4_direct.inc")):
         out = os.path.join(os.path.dirname(os.path.abspath(__file__)), name)
         txt = render()
         if "--check" in sys.argv:

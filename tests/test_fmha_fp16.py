@@ -208,6 +208,20 @@ def test_unusual_softmax_scales_on_the_hand_scheduled_kernel(scale):
     assert err <= (TOL_FP16 if scale < 0.5 else 2.5e-3) and not np.isnan(got).any()
 
 
+@pytest.mark.parametrize("B,S,H,D", [(1, 32768, 2, 128), (1, 32768, 3, 64), (1, 16384, 2, 256), (1, 65536, 1, 128)])
+def test_very_long_sequences(B, S, H, D):
+    # 256 to 1024 key tiles per work item: 64-bit tile addresses, row sums over tens of thousands of weights against one
+    # fixed reference point; every 1531st row of every head against the oracle
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    got, (qf, kf, vf) = _run(q, k, v)
+    ref = np.full(got.shape, np.nan, np.float32)
+    oracle.attention_f32(qf, kf, vf, bh_pairs=[(b, h) for b in range(B) for h in range(H)], row_start=5, row_step=1531, out=ref)
+    sel = ~np.isnan(ref)
+    err = max_abs(got[sel], ref[sel])
+    print(f"fp16 B={B} S={S} H={H} D={D}: checked {sel.sum()} elements, max-abs {err:.3e}")
+    assert sel.sum() >= (S // 1531) * H * D and err <= TOL_FP16 and np.isfinite(got).all()
+
+
 def test_config3_long_sequence_large_head_subset_check():
     # benchmark configuration 3: B=2 H=8 S=8192 D=256
     _subset_check(2, 8192, 8, 256)

@@ -500,3 +500,16 @@ def test_fast_e4m3_weights_second_pass(fast_weights, D):
     ref = oracle.attention_f32(qf, kf, vf)["O"]
     assert max_abs(got[0, 77, 1], vf[0, 1000, 1]) <= TOL_FP8
     assert not np.isnan(got).any() and max_abs(got, ref) <= TOL_FP8
+
+
+def test_very_long_sequence():
+    # 512 key tiles per work item on the hand-scheduled e4m3 kernel; every 1531st row of every head against the oracle
+    B, S, H, D = 1, 32768, 2, 128
+    q, k, v = pkg.testbed.qkv(B, S, H, D)
+    got, (qf, kf, vf) = _run(q, k, v)
+    ref = np.full(got.shape, np.nan, np.float32)
+    oracle.attention_f32(qf, kf, vf, bh_pairs=[(0, 0), (0, 1)], row_start=5, row_step=1531, out=ref)
+    sel = ~np.isnan(ref)
+    err = max_abs(got[sel], ref[sel])
+    print(f"e4m3 B={B} S={S} H={H} D={D}: checked {sel.sum()} elements, max-abs {err:.3e}")
+    assert err <= TOL_FP8 and np.isfinite(got).all()

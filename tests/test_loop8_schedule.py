@@ -52,7 +52,7 @@ class Checker:
         self.kptr, self.vptr = 3, 2
         self.next_item = {"s40": False, "s42": False}   # the pointer walks the next work item's tiles
         self.vm_pending = False                          # a load with a register destination is in flight
-        self.copied = {"s40": False, "s42": False}       # a copy has been issued since the pointer last moved
+        self.copied = {"s40": set(), "s42": set()}       # the parts of a tile copied since the pointer last moved
         self.kslot = {0: 0, 1: 1, 2: 2, 3: None}
         self.vslot = {0: 0, 1: 1, 2: None, 3: None}
         self.inflight = []    # copies issued since the last barrier: (kind, slot, tile)
@@ -69,8 +69,9 @@ class Checker:
             for h in range(2): self.put(g.KRD0 + 2 * s + h, ("krd", s, h), FOREVER, "init")
         for db in range(g.DB): self.put(g.VRD0 + db, ("vrd", db), FOREVER, "init")
         for i in range(8): self.put(g.ONES0 + i, ("ones", i), FOREVER, "init")
-        self.put(g.GOK, ("gok",), FOREVER, "init")
-        self.put(g.GOV, ("gov",), FOREVER, "init")
+        for i in range(g.ipw()):
+            self.put(g.GOK[i], ("gok", i), FOREVER, "init")
+            self.put(g.GOV[i], ("gov", i), FOREVER, "init")
 
     # ---- register file
     def put(self, r, tag, need, kind, pend=None):
@@ -207,9 +208,9 @@ class Checker:
                 gt = self.get(int(a[0][1:]), "vmem")
                 kind = "K" if self.m0 < g.V_ST0 else "V"
                 rel = self.m0 - (g.K_ST0 if kind == "K" else g.V_ST0)
-                slot = rel // g.K_TILE
+                slot, part = rel // g.K_TILE, (rel % g.K_TILE) // (g.NWAVES * 1024)
                 sp = "s40" if kind == "K" else "s42"
-                assert rel % g.K_TILE == 0 and slot < g.NSLOT and gt == ("gok" if kind == "K" else "gov",), ins
+                assert rel % (g.NWAVES * 1024) == 0 and part < g.ipw() and slot < g.NSLOT and gt == ("gok" if kind == "K" else "gov", part), ins
                 assert a[1] == ("s[40:41]" if kind == "K" else "s[42:43]")
                 t = self.kptr if kind == "K" else self.vptr
                 if self.next_item[sp]:
@@ -218,15 +219,15 @@ class Checker:
                 else:
                     assert t < self.n and slot == t % g.NSLOT, "copy of tile %d into slot %d (%s)" % (t, slot, ins)
                 assert (kind, slot) not in self.seg_reads, "%s slot %d read and then copied into in one barrier interval" % (kind, slot)
-                assert not self.copied[sp], "two copies of one tile"
-                self.copied[sp] = True
-                self.inflight.append((kind, slot, t))
+                assert part not in self.copied[sp], "two copies of one part of a tile"
+                self.copied[sp].add(part)
+                if part == 0: self.inflight.append((kind, slot, t))
                 (self.kslot if kind == "K" else self.vslot)[slot] = None
             elif op == "s_add_u32":
                 sp = a[0]
                 assert sp == a[1] and a[2] == "%[stride]" and sp in ("s40", "s42")
-                assert self.copied[sp], "pointer moved before the copy of the tile"
-                self.copied[sp] = False
+                assert self.copied[sp] == set(range(g.ipw())), "pointer moved before all copies of the tile"
+                self.copied[sp] = set()
                 if sp == "s40": self.kptr += 1
                 else: self.vptr += 1
             elif op == "s_mov_b64":
@@ -320,11 +321,12 @@ class Checker:
         assert self.idx - last_mfma > g.MIN_MFMA_TO_VALU
 
 
+@pytest.mark.parametrize("nwaves", [8, 4])
 @pytest.mark.parametrize("direct", [True, False])
 @pytest.mark.parametrize("n_tiles", [8, 12, 16, 32, 64, 128])
-def test_loop_is_correct_symbolically(n_tiles, direct):
+def test_loop_is_correct_symbolically(n_tiles, direct, nwaves):
     g = _gen()
-    g.DIRECT = direct
+    g.DIRECT, g.NWAVES = direct, nwaves
     c = Checker(g, n_tiles)
     c.run(g.program(n_tiles))
     c.finish()
@@ -362,4 +364,4 @@ def test_checker_catches_a_broken_schedule():
 
 def test_committed_include_is_the_generators_output():
     r = subprocess.run([sys.executable, os.path.join(CSRC, "gen_fmha_loop8.py"), "--check"])
-    assert r.returncode == 0, "fmha_fwd_loop8_d128.inc is stale: run gen_fmha_loop8.py"
+    assert r.returncode == 0, "fmha_fwd_loop8_d128*.inc are stale: run gen_fmha_loop8.py"
