@@ -888,8 +888,9 @@ constexpr bool fits(int sq, int skv) {
 // +9 %; at 128 items a tie, at 96 -4 %: there the 128-row tile's twice as many workgroups count).  Up to 256 items of 128
 // rows -- one round -- those head dims take the same loops in their 4-wave shape (128 rows, one wave per SIMD): +11..20 %
 // over the compiler-scheduled 128-row builds from 1024 keys on (2048 keys +12 %, 8192 +20 %, 1024 +2..6 %, 512 -5 %).
-// e4m3: from 160 items on (+13 %; at 128 items -11 %) and only while the last round of items keeps four fifths of the
-// workgroups busy (320 items -10 %, 384 items -6 %: the 128-row tile has twice the workgroups to even out the tail).
+// e4m3: the 8-wave shape from 160 items on (+8..13 %; at 128 items -11 %) and only while the last round of items keeps
+// four fifths of the workgroups busy (320 items -8 %, 384 items -5 %: the 128-row tile has twice the workgroups to even
+// out the tail); up to 256 items of 128 rows the 4-wave shape (+9..20 % over the compiler-scheduled 128-row build).
 template <class C>
 constexpr bool hand_loop_pays(long long items, int skv) {
   if (!C::QK8) return C::D == 256 ? skv >= 1024 : C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;

@@ -41,5 +41,6 @@ if [[ ${1:-fp16} == fp16 ]]; then
   sweep "--prec-type=1" 256 256 128x64/16h 8 32
 fi
 if [[ ${1:-fp8} == fp8 ]]; then
-  sweep "--prec-type=2 --gemm2-fp8=true" 128 4096 256x128/32h 4 8 10 12 16 20 24 28 32 64
+  sweep "--prec-type=2 --gemm2-fp8=true" 128 4096 "256x128/32h 128x128/32h" 2 4 6 8 10 12 16 20 24 28 32 64
+  sweep "--prec-type=2 --gemm2-fp8=true" 128 16384 "256x128/32h 128x128/32h" 1 2 4
 fi
