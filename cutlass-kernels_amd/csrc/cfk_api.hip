@@ -62,8 +62,8 @@ int check_fmha(const cfk_fmha_fwd_params *p, cfk::FmhaPlan *plan, bool need_poin
   // The kernels carry no masks, exactly like the reference (no bounds handling: fmha_forward.cu:361-372).
   if (p->seqlen_q % plan->block_m != 0)
     return fail(CFK_ERR_UNSUPPORTED, "seqlen_q %d is not a multiple of the query tile %d", p->seqlen_q, plan->block_m);
-  if (p->seqlen_kv % plan->block_n != 0)
-    return fail(CFK_ERR_UNSUPPORTED, "seqlen_kv %d is not a multiple of the key tile %d", p->seqlen_kv, plan->block_n);
+  if (p->seqlen_kv % plan->kv_multiple != 0)
+    return fail(CFK_ERR_UNSUPPORTED, "seqlen_kv %d is not a multiple of the key tile %d", p->seqlen_kv, plan->kv_multiple);
   const long long elems = bh * (long long)(p->seqlen_q > p->seqlen_kv ? p->seqlen_q : p->seqlen_kv) * p->head_dim;
   if (elems >= (1LL << 40)) return fail(CFK_ERR_UNSUPPORTED, "tensor too large");
   // the kernels address one batch slice with 32-bit byte offsets

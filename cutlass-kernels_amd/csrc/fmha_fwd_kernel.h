@@ -819,6 +819,7 @@ template <class C>
 void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
   p->block_m = C::BM;
   p->block_n = C::BN * C::SUB;
+  p->kv_multiple = C::ASM && !C::QK8 && C::D != 256 ? C::BN : C::BN * C::SUB;
   p->mfma = C::M16 ? 16 : 32;
   p->lds_bytes = C::LDS_BYTES;
   p->threads = C::T;
@@ -871,11 +872,13 @@ template <class... Cs>
 struct CfgList {};
 
 // the shapes an instantiation can run: whole query tiles, whole key steps (four key tiles per loop turn with the K
-// fragment prefetch and in the hand-scheduled loop, which also needs eight tiles to fill and drain; two with the
-// two-tile step)
+// fragment prefetch and in the e4m3 hand-scheduled loop; the hand-scheduled loops need eight tiles to fill and drain;
+// two tiles with the two-tile step)
 template <class C>
 constexpr bool fits(int sq, int skv) {
-  return sq % C::BM == 0 && skv % (C::BN * (C::KPRE || C::ASM ? 4 : C::SUB)) == 0 &&
+  // (the fp16 hand-scheduled builds at head dims 64 and 128 take up to three tiles behind the last group of four outside
+  // their loop)
+  return sq % C::BM == 0 && skv % (C::BN * (C::ASM && !C::QK8 && C::D != 256 ? 1 : C::KPRE || C::ASM ? 4 : C::SUB)) == 0 &&
          (!C::ASM || skv >= (C::QK8 ? 64 : 8) * C::BN);
 }
 

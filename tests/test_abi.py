@@ -160,7 +160,9 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 1, 8192, 8192, 256)          # (at head dim 256 from 1024 keys)
     assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 2, 1024, 1024, 256)
     assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 16, 64, 512, 512, 256)
-    assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 1, 40, 2048, 2048 + 64, 128)   # key length: whole 256s only
+    assert "kernel16p<128" in f.fmha_forward_kernel(f.CFK_FP16, 1, 40, 2048, 2048 + 64, 128)    # (a key length with a tile left over)
+    assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 1, 8, 8192, 8192 + 32, 256)    # (head dim 256: whole 128s only)
+    assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 16, 4096, 4096 + 64, 128)  # (e4m3: whole 256s only)
     assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 8, 4096, 4096, 128) == "fmha_fwd_kernel8p<128,64,4,2,1,1,0,0,2,0,0,1>"   # 128 items: the 4-wave shape
     assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 9, 4096, 4096, 128)      # 288 items of 128 rows, 144 of 256: neither
     assert "kernel8p<" in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 10, 4096, 4096, 128)         # 160

@@ -27,7 +27,7 @@ CASES = {
     "256x64/16": ["f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f16:2,256,1,128,64", "f16climb:1,512,2,128,448"],
     "128x128/16": ["f16:1,512,2,128", "f16:2,384,3,128,128", "f16:1,256,2,128,640", "f16climb:1,384,2,128"],
     "256x128/16": ["f16:1,512,2,128", "f16:1,768,2,128,384", "f16:2,256,1,128,128", "f16climb:1,512,2,128,768"],
-    # ... with the hand-scheduled main loop and persistent workgroups (key length a multiple of 256, at least 512): the
+    # ... with the hand-scheduled main loop and persistent workgroups (key length at least 512): the
     # scheduled loop (no taps), its fall-back for scores that leave the fp16 range of the weights (climbing keys), the
     # max-tracking loop that serves the taps; 2x16 heads x 2048 rows = 256 items (one per workgroup), 3x16x2048 = 384
     # (half of the workgroups take a second item), 5x16x1024 = 320 with climbing keys (fall-back, then a next item)
@@ -35,7 +35,11 @@ CASES = {
                     "f16ntclimb:1,512,2,128,768", "f16ntclimb:5,1024,16,128", "f16:1,512,2,128", "f16:3,2048,16,128", "f16climb:1,512,2,128,768",
                     # ... its head-dim-64 shape (row sum on the matrix pipe)
                     "f16nt:1,512,2,64", "f16nt:1,256,3,64,768", "f16nt:3,2048,16,64", "f16ntclimb:1,512,2,64,768", "f16ntclimb:5,1024,16,64",
-                    "f16:1,512,2,64", "f16climb:1,512,2,64,1024"],
+                    "f16:1,512,2,64", "f16climb:1,512,2,64,1024",
+                    # ... key lengths with one to three tiles behind the last group of four (taken outside the generated loop)
+                    "f16nt:1,512,2,128,576", "f16nt:2,2048,16,128,2240", "f16nt:1,256,3,128,640", "f16ntclimb:1,512,2,128,704",
+                    "f16nt:1,512,2,64,640", "f16nt:3,2048,16,64,2112", "f16ntclimb:1,512,2,64,576", "f16ntclimb:1,512,2,64,640",
+                    "f16ntclimb:1,512,2,128,576", "f16ntclimb:1,512,2,64,704"],   # (the spike key inside the loop's tiles, and behind them)
     # ... and its head-dim-256 shape (4 waves, one per SIMD, 32-key tiles; key length a multiple of 128, at least 256):
     # 3x6 heads x 2048 rows = 288 items of 128 rows (32 workgroups take a second one), climbing keys, taps
     "128x64/16h": ["f16nt:1,256,2,256", "f16nt:1,128,3,256,640", "f16nt:3,2048,6,256,512", "f16ntclimb:1,256,2,256,512",
@@ -46,7 +50,8 @@ CASES = {
                     "f16ntclimb:5,1024,8,128", "f16:1,256,2,128,512", "f16climb:1,256,2,128,768",
                     # ... and the head-dim-64 loop likewise
                     "f16nt:1,256,2,64,512", "f16nt:1,128,3,64,768", "f16nt:1,2048,20,64", "f16ntclimb:1,256,2,64,768", "f16ntclimb:5,1024,8,64",
-                    "f16:1,256,2,64,512", "f16climb:1,256,2,64,1024"],
+                    "f16:1,256,2,64,512", "f16climb:1,256,2,64,1024",
+                    "f16nt:1,256,2,128,1088", "f16nt:1,2048,20,128,1216", "f16nt:1,256,2,64,1216", "f16ntclimb:1,256,2,64,1088", "f16ntclimb:1,128,2,128,576"],
     # the e4m3 build with the hand-scheduled loop and persistent workgroups (key length a multiple of 256, from 4096): the
     # scheduled loop, 4352 keys (an odd number of loop turns), 2x10 heads x 4096 rows = 320 items (a quarter of the
     # workgroups take a second one), climbing keys (the vote, the max-tracking loop, then a next item: 5x13x1024 rows = 260)
@@ -101,16 +106,16 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     def lds(wish):
         env = dict(os.environ, CFK_FMHA_TILE=wish)
         return subprocess.run([sys.executable, "-c", lds_code], env=env, capture_output=True, text=True, check=True).stdout.strip()
-    assert lds("256x128/16h") == "163840 (128, 64, 65536)"    # key length 384: not a multiple of 256, the wish is ignored
+    assert lds("256x128/16h") == "163840 (128, 64, 65536)"    # key length 384: fewer than eight tiles, the wish is ignored
     assert lds("256x128/16") == "131072 (256, 128, 131072)"
     assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:2] == (256, 128)  # big problem: automatic choice
-    assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 1984, 128)[:2] == (256, 64)   # ... key length not a multiple of 128
+    assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 1984, 128)[:2] == (256, 128)  # ... also with tiles left over behind the last four
     # ... on 16x16x32 MFMAs for fp16; problems with fewer work items than half the CUs (head dims 64, 128) and e4m3 stay on 32x32
     assert f.fmha_forward_mfma(f.CFK_FP16, 8, 16, 2048, 2048, 128) == 16
     assert f.fmha_forward_mfma(f.CFK_FP16, 4, 32, 4096, 4096, 64) == 16
     assert f.fmha_forward_plan(f.CFK_FP16, 4, 32, 4096, 4096, 64)[:2] == (256, 128)      # hand-scheduled
     assert f.fmha_forward_kernel(f.CFK_FP16, 4, 32, 4096, 4096, 64) == "fmha_fwd_kernel16p<64,64,8,2,0,0,0,0,2,0,1,1>"
-    assert f.fmha_forward_plan(f.CFK_FP16, 4, 32, 4096, 4032, 64)[:2] == (128, 64)       # key length % 256 != 0
+    assert f.fmha_forward_plan(f.CFK_FP16, 4, 32, 4096, 4032, 64)[:2] == (256, 128)      # ... also with tiles left over
     assert f.fmha_forward_mfma(f.CFK_FP16, 2, 4, 1536, 512, 128) == 32
     assert f.fmha_forward_kernel(f.CFK_FP16, 1, 8, 512, 512, 64) == "fmha_fwd_kernel_ks<64,8>"      # benchmark configuration 1
     assert f.fmha_forward_kernel(f.CFK_FP16, 2, 4, 512, 512, 128) == "fmha_fwd_kernel_ks<128,8>"
