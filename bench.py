@@ -68,6 +68,9 @@ WORKLOADS = {
     # fifth of the weights are then one e4m3 step off the correctly rounded one)
     "cfg4_fast_weights": dict(kind="fmha", dtype="f8", B=4, H=16, S=4096, D=128, scale=None, fast_weights=True),
     "d64_f8_fast_weights": dict(kind="fmha", dtype="f8", B=4, H=32, S=4096, D=64, scale=None, fast_weights=True),
+    # one sequence, 256 work items of 128 rows: what the 4-wave shapes of the hand-scheduled loops are for
+    "b1_f16": dict(kind="fmha", dtype="f16", B=1, H=16, S=2048, D=128, scale=None),
+    "b1_f8": dict(kind="fmha", dtype="f8", B=1, H=8, S=4096, D=128, scale=None),
     "d64_f16": dict(kind="fmha", dtype="f16", B=4, H=32, S=4096, D=64, scale=None),   # the reference sweep's head size 64
     "d64_f8": dict(kind="fmha", dtype="f8", B=4, H=32, S=4096, D=64, scale=None),
     "gemm_f32": dict(kind="gemm", dtype="f32", M=8192, N=8192, K=8192, max_steps=50),  # the CuTe example's type 1
@@ -78,6 +81,8 @@ NAMES = {
     "cfg3": "fmha_fwd fp16 B=2 H=8 S=8192 D=256 non-causal",
     "cfg4": "fmha_fwd fp8-e4m3 B=4 H=16 S=4096 D=128 non-causal, per-tensor amax scales, V [B,S,H,D]",
     "cfg5": "gemm fp16 M=N=K=8192 TN fp32-accumulate",
+    "b1_f16": "fmha_fwd fp16 B=1 H=16 S=2048 D=128 non-causal (one sequence: 256 work items of 128 rows)",
+    "b1_f8": "fmha_fwd fp8-e4m3 B=1 H=8 S=4096 D=128 non-causal (one sequence: 256 work items of 128 rows)",
     "cfg4_climb": "fmha_fwd fp8-e4m3 B=4 H=16 S=4096 D=128, keys scaled 1..4 along the key axis and one key x8 (scores climb: "
                   "every workgroup takes the second, max-tracking pass)",
     "cfg4_climb_one_pass": "... the same data with cfk_set_option(CFK_OPT_PREDICTABLE_LATENCY, 1): max-tracking pass only",
@@ -158,7 +163,7 @@ def run_workload(pkg, name, steps, warmup):
     fn, flop, keep = (_make_fmha if w["kind"] == "fmha" else _make_gemm)(pkg, w)
     # configuration 1 is a 9-microsecond kernel: the reference's protocol (mean over back-to-back launches) needs
     # many more of them for a stable mean
-    n = steps * 20 if name == "cfg1" else min(steps, w.get("max_steps", steps))
+    n = steps * 20 if name == "cfg1" else steps * 4 if name.startswith("b1_") else min(steps, w.get("max_steps", steps))
     if w.get("one_pass"):
         pkg.fmha.set_option(pkg.fmha.CFK_OPT_PREDICTABLE_LATENCY, 1)
     if w.get("fast_weights"):
