@@ -60,8 +60,8 @@ int check_fmha(const cfk_fmha_fwd_params *p, cfk::FmhaPlan *plan, bool need_poin
                                      : cfk::plan_fmha_fp8(p->head_dim, p->seqlen_q, p->seqlen_kv, (int)bh, p->v_layout, tap, plan);
   if (!ok) return fail(CFK_ERR_UNSUPPORTED, "no kernel for dtype %d head dim %d v_layout %d", p->dtype, p->head_dim, p->v_layout);
   // The kernels carry no masks, exactly like the reference (no bounds handling: fmha_forward.cu:361-372).
-  if (p->seqlen_q % plan->block_m != 0)
-    return fail(CFK_ERR_UNSUPPORTED, "seqlen_q %d is not a multiple of the query tile %d", p->seqlen_q, plan->block_m);
+  if (p->seqlen_q % plan->q_multiple != 0)
+    return fail(CFK_ERR_UNSUPPORTED, "seqlen_q %d is not a multiple of %d (query tile %d)", p->seqlen_q, plan->q_multiple, plan->block_m);
   if (p->seqlen_kv % plan->kv_multiple != 0)
     return fail(CFK_ERR_UNSUPPORTED, "seqlen_kv %d is not a multiple of the key tile %d", p->seqlen_kv, plan->kv_multiple);
   const long long elems = bh * (long long)(p->seqlen_q > p->seqlen_kv ? p->seqlen_q : p->seqlen_kv) * p->head_dim;

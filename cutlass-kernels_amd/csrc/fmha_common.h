@@ -32,6 +32,7 @@ bool fast_e4m3_weights();
 
 struct FmhaPlan {
   int32_t block_m, block_n, lds_bytes, threads, grid;
+  int32_t q_multiple;   // what the query length has to be a multiple of (block_m, or 32 where the last tile may be partly filled)
   int32_t kv_multiple;  // what the key length has to be a multiple of (block_n, or one key tile where the kernel has a tail)
   int32_t mfma;  // 32: 32x32 MFMA build, 16: 16x16x32 build
   char kernel[80];  // the instantiation, as profilers print it without namespaces: fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>

@@ -176,7 +176,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, g = lane >> 5;
 
-  const int q_blocks = a.Sq / C::BM;
+  const int q_blocks = (a.Sq + C::BM - 1) / C::BM;   // the last query tile may be partly filled: whole waves of 32 rows
   const int tile = xcd_remap(blockIdx.x, gridDim.x);
   const int bh = tile / q_blocks;
   const int qb = tile - bh * q_blocks;
@@ -189,7 +189,10 @@ fmha_fwd_kernel(const FmhaArgs a) {
   const char *Vp = C::VT ? (const char *)a.v + ((int64_t)b * D * a.H + h) * a.Skv
                          : (const char *)a.v + (((int64_t)b * a.Skv * a.H + h) * D) * VES;
   _Float16 *Op = (_Float16 *)a.o + ((int64_t)b * a.Sq * a.H + h) * D;
-  const int q0 = qb * C::BM + wave * 32;
+  // A wave behind the last query row still copies its share of every K/V tile and meets every barrier; it computes on
+  // the last 32 rows (loads stay in bounds) and stores nothing.
+  const bool live = qb * C::BM + wave * 32 < a.Sq;
+  const int q0 = live ? qb * C::BM + wave * 32 : a.Sq - 32;
   const int n_tiles = a.Skv / BN;
   const float c_log2 = a.scale_log2;
   // global row pitch in bytes
@@ -343,7 +346,7 @@ fmha_fwd_kernel(const FmhaArgs a) {
   };
   // Row max of a finished S tile and the deferred rescale (online_softmax.h:123-165).  The branch is wave-uniform.
   auto row_max_and_rescale = [&](const f32x16 (&sacc)[KB], int jt) __attribute__((always_inline)) {
-    if constexpr (C::TAP_S) {  // the reference's -DCOPYOUTMM0 dump (fmha_consumer.h:31-42), here already scaled
+    if (C::TAP_S && live) {  // the reference's -DCOPYOUTMM0 dump (fmha_consumer.h:31-42), here already scaled
       float *srow = a.s_tap + (((int64_t)b * a.H + h) * a.Sq + q0 + r) * (int64_t)a.Skv + (int64_t)jt * BN;
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
@@ -730,10 +733,10 @@ fmha_fwd_kernel(const FmhaArgs a) {
     for (int pass = 0; pass < 32 / RPP; ++pass) {
       const int row = pass * RPP + orow_l;
       const int4v val = *(const int4v *)(ot + row * C::O_PITCH + ochunk * 16);
-      *(int4v *)(Op + (int64_t)(q0 + row) * ld + ochunk * 8) = val;
+      if (live) *(int4v *)(Op + (int64_t)(q0 + row) * ld + ochunk * 8) = val;
     }
   }
-  if (a.row_max || a.row_sum) {
+  if (live && (a.row_max || a.row_sum)) {
     const float m_true = fmaxf(m_lane, __shfl_xor(m_lane, 32, 64)) * c_log2;
     if (g == 0) {
       const int64_t si = ((int64_t)b * a.H + h) * a.Sq + qrow;
@@ -764,6 +767,12 @@ struct DirectCfg : C {
 };
 template <class C>
 constexpr bool has_direct_build = C::PV8 && C::D <= 128 && !C::TAP_S && !C::KSPLIT;
+
+// What the query length has to be a multiple of: the compiler-scheduled 32x32 kernel (fmha_fwd_kernel) takes a last
+// query tile filled to a whole number of waves (32 rows each), the other kernels whole tiles.  (The reference: whole
+// tiles of its compile-time 64 or 128 rows, src/fmha-pipeline/shared_storage.h:4-15.)
+template <class C>
+constexpr int q_multiple = !C::KSPLIT && !C::ASM && !C::M16 ? 32 : C::BM;
 
 template <class C>
 constexpr auto fmha_kernel_of() {
@@ -803,7 +812,7 @@ template <class C>
 hipError_t launch_fmha_cfg(const FmhaArgs &a, hipStream_t s) {
   const hipError_t e = prepare_fmha_cfg<C>();
   if (e != hipSuccess) return e;
-  const int items = a.B * a.H * (a.Sq / C::BM);
+  const int items = a.B * a.H * ((a.Sq + C::BM - 1) / C::BM);
   const int grid = C::ASM ? persistent_grid(items) : items;
   if constexpr (has_direct_build<C>) {
     if (a.direct_p != 0) {
@@ -820,10 +829,11 @@ void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
   p->block_m = C::BM;
   p->block_n = C::BN * C::SUB;
   p->kv_multiple = C::ASM && !C::QK8 && C::D != 256 ? C::BN : C::BN * C::SUB;
+  p->q_multiple = q_multiple<C>;
   p->mfma = C::M16 ? 16 : 32;
   p->lds_bytes = C::LDS_BYTES;
   p->threads = C::T;
-  p->grid = bh * (sq / C::BM);
+  p->grid = bh * ((sq + C::BM - 1) / C::BM);
   if constexpr (C::KSPLIT) {
     snprintf(p->kernel, sizeof p->kernel, "fmha_fwd_kernel_ks<%d,%d>", C::D, C::NWAVES);
     return;
@@ -871,14 +881,14 @@ inline TileWish tile_wish() {
 template <class... Cs>
 struct CfgList {};
 
-// the shapes an instantiation can run: whole query tiles, whole key steps (four key tiles per loop turn with the K
+// the shapes an instantiation can run: whole query tiles (fmha_fwd_kernel: whole waves), whole key steps (four key tiles per loop turn with the K
 // fragment prefetch and in the e4m3 hand-scheduled loop; the hand-scheduled loops need eight tiles to fill and drain;
 // two tiles with the two-tile step)
 template <class C>
 constexpr bool fits(int sq, int skv) {
   // (the fp16 hand-scheduled builds at head dims 64 and 128 take up to three tiles behind the last group of four outside
   // their loop)
-  return sq % C::BM == 0 && skv % (C::BN * (C::ASM && !C::QK8 && C::D != 256 ? 1 : C::KPRE || C::ASM ? 4 : C::SUB)) == 0 &&
+  return sq % q_multiple<C> == 0 && skv % (C::BN * (C::ASM && !C::QK8 && C::D != 256 ? 1 : C::KPRE || C::ASM ? 4 : C::SUB)) == 0 &&
          (!C::ASM || skv >= (C::QK8 ? 64 : 8) * C::BN);
 }
 

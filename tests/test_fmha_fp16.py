@@ -103,14 +103,14 @@ def test_row_max_and_row_sum_taps():
     np.testing.assert_allclose(1.0 / rs.cpu().numpy(), r["inv_sum"], rtol=1e-4)
 
 
-@pytest.mark.parametrize("D", [64, 128, 256])
-def test_score_tap(D):
+@pytest.mark.parametrize("D,S", [(64, 256), (128, 256), (256, 256), (128, 160), (256, 96)])
+def test_score_tap(D, S):
     # the reference's gemm-check-1 (fmha_forward.cu:640-653): pre-softmax scores against the oracle's, exact
-    # products of fp16 values accumulated in fp32
+    # products of fp16 values accumulated in fp32 (160 and 96 query rows: a last query tile that is partly filled)
     import torch
-    B, S, H = 2, 256, 2
-    q, k, v = pkg.testbed.qkv(B, S, H, D)
-    sc = torch.full((B, H, S, S), -1.0, dtype=torch.float32, device="cuda:0")
+    B, H, Skv = 2, 2, 256
+    q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=Skv)
+    sc = torch.full((B, H, S, Skv), -1.0, dtype=torch.float32, device="cuda:0")
     got, (qf, kf, vf) = _run(q, k, v, scores=sc)
     r = oracle.attention_f32(qf, kf, vf, want_scores=True)
     assert max_abs(got, r["O"]) <= TOL_FP16

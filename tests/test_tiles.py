@@ -14,13 +14,17 @@ from _util import ERRPCT_FP16, ERRPCT_FP8, ROOT, TOL_FP16, TOL_FP8, pkg
 CASES = {
     "128x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f16climb:1,256,2,128,384", "f8:1,2048,2,64", "f8:1,2048,2,128", "f8:1,2048,1,256",
                "f8climb:1,256,2,64,4096", "f8climb:1,256,2,128,4096", "f8climb:1,128,1,256,4096", "f8:1,4096,1,64", "f8:1,4096,1,128", "f8:1,4096,1,256",
-               "hyb:1,512,2,64", "hyb:1,512,2,128", "f16:1,256,2,256", "f16climb:1,256,1,256,192"],
-    "256x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f8:1,2048,2,128", "hyb:1,512,2,128",
+               "hyb:1,512,2,64", "hyb:1,512,2,128", "f16:1,256,2,256", "f16climb:1,256,1,256,192",
+               # ... a last query tile filled to a whole number of waves (32 rows each)
+               "f16:2,160,2,64,192", "f16:2,288,3,128,192", "f16:2,160,2,256,128", "f16climb:2,160,2,128,384", "f8:2,160,2,64,2048",
+               "f8:2,288,2,128,2048", "f8:2,96,1,256,2048", "f8climb:2,160,2,128,4096", "hyb:2,160,2,64,512", "hyb:2,96,2,128,512"],
+    "256x64": ["f16:2,288,2,128,320", "f8:2,320,2,128,2048", "hyb:2,416,2,128,512",
+               "f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128", "f16:1,512,2,128,320", "f8:1,2048,2,128", "hyb:1,512,2,128",
                "f8climb:1,256,2,128,4096", "f8:1,4096,1,128"],
-    "128x128": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,384,2,128", "f8:1,2048,2,64", "f8:1,2048,2,128",
+    "128x128": ["f16:2,224,2,64,256", "f8:2,160,2,64,2048", "hyb:2,160,2,64,512", "f16:1,512,2,64", "f16:1,512,2,128", "f16:1,384,2,128", "f8:1,2048,2,64", "f8:1,2048,2,128",
                 "f8:1,2048,1,256", "hyb:1,512,2,64", "f8climb:1,256,2,64,4096", "f8climb:1,256,2,128,4096", "f8climb:1,128,1,256,4096", "f8:1,4096,1,64", "f8:1,4096,1,128"],
-    "256x128": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128,384", "f8:1,2048,2,128", "hyb:1,512,2,128", "f8climb:1,256,2,128,4096", "f8:1,4096,1,128"],
-    "128x32": ["f16:1,256,2,256", "hyb:1,256,2,256"],
+    "256x128": ["f16:2,416,2,128,384", "f8:2,1184,2,128,2048", "f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128,384", "f8:1,2048,2,128", "hyb:1,512,2,128", "f8climb:1,256,2,128,4096", "f8:1,4096,1,128"],
+    "128x32": ["f16:1,256,2,256", "hyb:1,256,2,256", "f16:2,96,2,256,256", "hyb:2,224,2,256,256"],
     # the fp16 builds on 16x16x32 MFMAs
     "128x64/16": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:2,384,3,128,192", "f16:1,256,2,64,64", "f16climb:1,256,2,64,512",
                   "f16climb:1,384,2,128", "f16climb:1,128,1,128,64"],
@@ -81,8 +85,9 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     # medium problems: 128-row tiles; small ones (the last: 128 workgroups of 32 rows fit on the chip at once): fp16 at head
     # dims 64 and 128 takes 32-row workgroups whose waves split the keys
     assert plans(None) == "(128, 64) (128, 32) (128, 64) (128, 64) (32, 64)"
-    assert plans("256x128") == "(256, 128) (128, 32) (256, 128) (128, 64) (256, 128)"     # no such tile at head dim 256; 384 % 256 != 0
-    assert plans("large") == "(256, 64) (128, 32) (256, 64) (128, 64) (256, 64)"
+    # no such tile at head dim 256; 384 query rows: the second 256-row tile is half filled (whole waves of 32 rows)
+    assert plans("256x128") == "(256, 128) (128, 32) (256, 128) (256, 128) (256, 128)"
+    assert plans("large") == "(256, 64) (128, 32) (256, 64) (256, 64) (256, 64)"
     assert plans("128x128") == "(128, 128) (128, 32) (128, 128) (128, 128) (128, 128)"
     assert plans("32x64") == "(32, 64) (128, 32) (128, 64) (32, 64) (32, 64)"              # fp16 at head dims 64 / 128 only
     # the MFMA shape suffix: served for fp16 at head dims 64/128 only (e4m3 and head dim 256 ignore the wish)
