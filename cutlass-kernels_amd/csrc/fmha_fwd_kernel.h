@@ -768,11 +768,12 @@ struct DirectCfg : C {
 template <class C>
 constexpr bool has_direct_build = C::PV8 && C::D <= 128 && !C::TAP_S && !C::KSPLIT;
 
-// What the query length has to be a multiple of: the compiler-scheduled 32x32 kernel (fmha_fwd_kernel) takes a last
-// query tile filled to a whole number of waves (32 rows each), the other kernels whole tiles.  (The reference: whole
+// What the query length has to be a multiple of: the compiler-scheduled 32x32 kernel (fmha_fwd_kernel) and the
+// hand-scheduled fp16 kernel (fmha_fwd_kernel16p) take a last query tile filled to a whole number of waves (32 rows
+// each), the other kernels whole tiles.  (The reference: whole
 // tiles of its compile-time 64 or 128 rows, src/fmha-pipeline/shared_storage.h:4-15.)
 template <class C>
-constexpr int q_multiple = !C::KSPLIT && !C::ASM && !C::M16 ? 32 : C::BM;
+constexpr int q_multiple = !C::KSPLIT && (C::ASM ? !C::QK8 : !C::M16) ? 32 : C::BM;
 
 template <class C>
 constexpr auto fmha_kernel_of() {
@@ -922,7 +923,7 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish
   auto try_one = [&](auto c) {
     using C = decltype(c);
     if (done || !fits<C>(sq, skv)) return;
-    const bool by_size = C::ASM ? hand_loop_pays<C>(bh * (sq / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
+    const bool by_size = C::ASM ? hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
     if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : !by_size)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
     if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;

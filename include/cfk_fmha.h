@@ -58,9 +58,9 @@ typedef struct cfk_fmha_fwd_params {
                         without -DGEMM2FP8 (fmha_forward.cu:446-450)                                            */
   int32_t batch;     /* BATCH                                                                                 */
   int32_t heads;     /* NUMHEADS                                                                              */
-  int32_t seqlen_q;  /* SEQLEN: multiple of 32.  Whole tiles of 128 or 256 query rows get the fastest kernels; other
-                        lengths a kernel whose last query tile is filled to a whole number of 32-row waves (the
-                        reference: whole tiles of its compile-time 64 or 128 rows, shared_storage.h:4-15)       */
+  int32_t seqlen_q;  /* SEQLEN: multiple of 32; a last query tile (128 or 256 rows) may be filled to a whole number
+                        of 32-row waves (the reference: whole tiles of its compile-time 64 or 128 rows,
+                        shared_storage.h:4-15)                                                                */
   int32_t seqlen_kv; /* KEYLEN: multiple of 64 (32 for fp16 V at head_dim 256); cfk_fmha_forward_plan reports the
                         key tile actually chosen                                                              */
   int32_t head_dim;  /* HEADDIM: 64, 128 or 256 (fmha_forward.cu:746-761)                                     */

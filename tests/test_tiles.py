@@ -43,11 +43,15 @@ CASES = {
                     # ... key lengths with one to three tiles behind the last group of four (taken outside the generated loop)
                     "f16nt:1,512,2,128,576", "f16nt:2,2048,16,128,2240", "f16nt:1,256,3,128,640", "f16ntclimb:1,512,2,128,704",
                     "f16nt:1,512,2,64,640", "f16nt:3,2048,16,64,2112", "f16ntclimb:1,512,2,64,576", "f16ntclimb:1,512,2,64,640",
-                    "f16ntclimb:1,512,2,128,576", "f16ntclimb:1,512,2,64,704"],   # (the spike key inside the loop's tiles, and behind them)
+                    "f16ntclimb:1,512,2,128,576", "f16ntclimb:1,512,2,64,704",    # (the spike key inside the loop's tiles, and behind them)
+                    # ... a last query tile filled to a whole number of waves: 2x16 heads x 2016 rows, 3x16x2016 (second items)
+                    "f16nt:2,416,3,128,768", "f16nt:2,2016,16,128,2048", "f16nt:3,2016,16,64,2112", "f16ntclimb:2,288,2,128,768",
+                    "f16ntclimb:2,352,2,64,640", "f16:2,416,2,128,768"],
     # ... and its head-dim-256 shape (4 waves, one per SIMD, 32-key tiles; key length a multiple of 128, at least 256):
     # 3x6 heads x 2048 rows = 288 items of 128 rows (32 workgroups take a second one), climbing keys, taps
     "128x64/16h": ["f16nt:1,256,2,256", "f16nt:1,128,3,256,640", "f16nt:3,2048,6,256,512", "f16ntclimb:1,256,2,256,512",
-                   "f16ntclimb:3,1024,12,256,256", "f16:1,256,2,256,384", "f16climb:1,256,2,256,512"],
+                   "f16ntclimb:3,1024,12,256,256", "f16:1,256,2,256,384", "f16climb:1,256,2,256,512",
+                   "f16nt:2,160,2,256,512", "f16nt:3,2016,6,256,512", "f16ntclimb:2,224,3,256,512", "f16:2,96,2,256,384"],   # (partly filled last tile)
     # ... and the head-dim-128 loop for 128 query rows (4 waves, one per SIMD, O in accumulation registers): 1x20 heads x
     # 2048 rows = 320 items (64 workgroups take a second one), climbing keys, taps
     "128x128/16h": ["f16nt:1,256,2,128,512", "f16nt:1,128,3,128,768", "f16nt:1,2048,20,128", "f16nt:2,384,3,128,1024", "f16ntclimb:1,256,2,128,768",
@@ -55,7 +59,8 @@ CASES = {
                     # ... and the head-dim-64 loop likewise
                     "f16nt:1,256,2,64,512", "f16nt:1,128,3,64,768", "f16nt:1,2048,20,64", "f16ntclimb:1,256,2,64,768", "f16ntclimb:5,1024,8,64",
                     "f16:1,256,2,64,512", "f16climb:1,256,2,64,1024",
-                    "f16nt:1,256,2,128,1088", "f16nt:1,2048,20,128,1216", "f16nt:1,256,2,64,1216", "f16ntclimb:1,256,2,64,1088", "f16ntclimb:1,128,2,128,576"],
+                    "f16nt:1,256,2,128,1088", "f16nt:1,2048,20,128,1216", "f16nt:1,256,2,64,1216", "f16ntclimb:1,256,2,64,1088", "f16ntclimb:1,128,2,128,576",
+                    "f16nt:2,160,3,128,1088", "f16nt:1,2016,20,64,1216", "f16ntclimb:2,224,2,128,768", "f16:2,96,2,64,512"],   # (partly filled last tile)
     # the e4m3 build with the hand-scheduled loop and persistent workgroups (key length a multiple of 256, from 4096): the
     # scheduled loop, 4352 keys (an odd number of loop turns), 2x10 heads x 4096 rows = 320 items (a quarter of the
     # workgroups take a second one), climbing keys (the vote, the max-tracking loop, then a next item: 5x13x1024 rows = 260)
