@@ -769,11 +769,11 @@ template <class C>
 constexpr bool has_direct_build = C::PV8 && C::D <= 128 && !C::TAP_S && !C::KSPLIT;
 
 // What the query length has to be a multiple of: the compiler-scheduled 32x32 kernel (fmha_fwd_kernel) and the
-// hand-scheduled fp16 kernel (fmha_fwd_kernel16p) take a last query tile filled to a whole number of waves (32 rows
-// each), the other kernels whole tiles.  (The reference: whole
+// hand-scheduled kernels (fmha_fwd_kernel16p, fmha_fwd_kernel8p) take a last query tile filled to a whole number of
+// waves (32 rows each), the other kernels whole tiles.  (The reference: whole
 // tiles of its compile-time 64 or 128 rows, src/fmha-pipeline/shared_storage.h:4-15.)
 template <class C>
-constexpr int q_multiple = !C::KSPLIT && (C::ASM ? !C::QK8 : !C::M16) ? 32 : C::BM;
+constexpr int q_multiple = !C::KSPLIT && (C::ASM || !C::M16) ? 32 : C::BM;
 
 template <class C>
 constexpr auto fmha_kernel_of() {
