@@ -890,7 +890,7 @@ constexpr bool fits(int sq, int skv) {
   // (the fp16 hand-scheduled builds at head dims 64 and 128 take up to three tiles behind the last group of four outside
   // their loop)
   return sq % q_multiple<C> == 0 && skv % (C::BN * (C::ASM && !C::QK8 && C::D != 256 ? 1 : C::KPRE || C::ASM ? 4 : C::SUB)) == 0 &&
-         (!C::ASM || skv >= (C::QK8 ? 64 : 8) * C::BN);
+         (!C::ASM || skv >= 8 * C::BN);
 }
 
 // Where a hand-scheduled persistent build (one workgroup per CU, each walking its share of the work items) beats the
@@ -905,10 +905,20 @@ constexpr bool fits(int sq, int skv) {
 // e4m3: the 8-wave shape from 160 items on (+8..13 %; at 128 items -11 %) and only while the last round of items keeps
 // four fifths of the workgroups busy (320 items -8 %, 384 items -5 %: the 128-row tile has twice the workgroups to even
 // out the tail); up to 256 items of 128 rows the 4-wave shape (+9..20 % over the compiler-scheduled 128-row build).
+// Those are the figures from 4096 keys on.  At 512 to 3072 keys the compiler-scheduled e4m3 builds lose more to their
+// prologue and epilogue: there the 4-wave shape is +19..50 % up to 256 items of 128 rows and the 8-wave shape +7..38 % at
+// every item count above (576 items of 128 rows +7..10 %, 1024 and more +22..28 %).
 template <class C>
 constexpr bool hand_loop_pays(long long items, int skv) {
   if (!C::QK8) return C::D == 256 ? skv >= 1024 : C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;
+  // (e4m3: the hand-scheduled loop sets its reference point from the first key tile, so a row's largest weight is not an
+  // exact power of two as it is for a reference point that follows the running max; over few keys the rounding of that
+  // weight does not average out -- the reference's error percentage, fmha_forward.cu:638-639 with its limit of 0.001 %,
+  // reads 0.0001 % at 3072 keys, 0.0003..0.0008 % at 2048, 0.03 % at 1024 (0.005 % for the max-tracking pass) -- so
+  // shorter key lengths take it only by wish (CFK_FMHA_TILE=256x128/32h or 128x128/32h: +19..50 % there))
+  if (skv < 3072) return false;
   if (C::BM == 128) return items <= 256;   // (the 4-wave shape: one round of 128-row items)
+  if (skv < 4096) return items > 128;      // (shorter key lengths: wherever the 4-wave shape does not apply)
   const long long rounds = (items + 255) / 256;
   return items >= 160 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
 }
