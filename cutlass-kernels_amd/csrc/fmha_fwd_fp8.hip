@@ -14,8 +14,9 @@ using C128_128x64 = FmhaCfg<128, 64, 4, 2, true, true>;
 using C128_256x64 = FmhaCfg<128, 64, 8, 2, true, true>;
 using C128_128x128 = FmhaCfg<128, 64, 4, 2, true, true, false, false, 2>;
 using C128_256x128 = FmhaCfg<128, 64, 8, 2, true, true, false, false, 2>;
-// ... with the hand-scheduled main loop and persistent workgroups (fmha_fwd_kernel8p.h); key sequences from 4096: below,
-// e4m3 weights run the max-tracking pass only (cfk_api.hip), which this build would do in a loop that is not pipelined
+// ... with the hand-scheduled main loop and persistent workgroups (fmha_fwd_kernel8p.h); key sequences from 3072 (by wish
+// from 512): below, e4m3 weights run the max-tracking pass only (cfk_api.hip, hand_loop_pays in fmha_fwd_kernel.h),
+// which this build would do in a loop that is not pipelined
 using A128_256x128 = FmhaCfg<128, 64, 8, 2, true, true, false, false, 2, 0, false, true>;
 using A128_128x128 = FmhaCfg<128, 64, 4, 2, true, true, false, false, 2, 0, false, true>;   // the same loop, 4 waves, one per SIMD
 using C256_128x64 = FmhaCfg<256, 64, 4, 1, true, true>;

@@ -66,10 +66,14 @@ def _load_dump(d):
 @pytest.mark.gpu
 @pytest.mark.parametrize("prec,head,extra", [(1, 64, []), (1, 128, ["--num-cuda-streams=2"]), (1, 256, []),
                                              (2, 128, []), (2, 128, ["--fp8-scales=amax"]), (2, 64, []), (2, 256, []), (2, 128, ["--gemm2-fp8=false"]),
-                                             (2, 128, ["--v-layout=bdhs"]), (2, 64, ["--v-layout=bdhs", "--fp8-scales=amax"])])
+                                             (2, 128, ["--v-layout=bdhs"]), (2, 64, ["--v-layout=bdhs", "--fp8-scales=amax"]),
+                                             # sequence lengths that leave the last 128-row query tile partly filled
+                                             (1, 128, ["seq=1088"]), (1, 256, ["seq=608"]), (2, 128, ["seq=4160"])])
 def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
     # fp8 needs the reference's own sequence length for its percentage criterion; fp16 passes at any length
     seq = 4096 if prec == 2 else 512   # (e4m3 P: the two-pass path starts at 4096 keys)
+    seq = next((int(e[4:]) for e in extra if e.startswith("seq=")), seq)
+    extra = [e for e in extra if not e.startswith("seq=")]
     out = _run(f"--prec-type={prec}", "--batch-size=2", f"--dim-size={2 * head}", f"--head-size={head}",
                f"--seq-length={seq}", "--iterations=3", "--reference-check=true", "--verify-all=true",
                f"--dump-dir={tmp_path}", *extra).stdout
