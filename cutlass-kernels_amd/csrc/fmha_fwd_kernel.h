@@ -957,8 +957,6 @@ void select_tile(int sq, int skv, int bh, F &&f) {
   static const bool no_hand = [] { const char *e = getenv("CFK_FMHA_HANDLOOP"); return e && e[0] == '0'; }();
   // (the hand-scheduled build is a two-pass kernel: not for callers that asked for a data-independent run time)
   if (first_fit(Auto{}, sq, skv, bh, size, TileWish{0, 0, 0, no_hand || predictable_latency() ? -1 : 0}, f)) return;
-  // query lengths that only the 32-row (key-split) build divides
-  if (first_fit(Auto{}, sq, skv, bh, 0, TileWish{32, 0, 0, 0}, f)) return;
   f(Fallback{});
 }
 
