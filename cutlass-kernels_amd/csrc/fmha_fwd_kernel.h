@@ -933,7 +933,11 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish
   auto try_one = [&](auto c) {
     using C = decltype(c);
     if (done || !fits<C>(sq, skv)) return;
-    const bool by_size = C::ASM ? hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
+    // (a 256-row tile whose last waves lie behind the last query row idles them: worth it while the hand-scheduled loop's
+    // lead over a 128-row build -- 20..30 % for fp16, 7..9 % for e4m3 -- outweighs the idle share of the rows)
+    const long long padded = (long long)((sq + C::BM - 1) / C::BM) * C::BM;
+    const bool tight = C::BM <= 128 || (padded - sq) * (C::QK8 ? 16 : 4) <= padded;
+    const bool by_size = C::ASM ? tight && hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
     if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : !by_size)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
     if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;

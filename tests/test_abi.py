@@ -161,6 +161,12 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 2, 1024, 1024, 256)
     assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 16, 64, 512, 512, 256)
     assert "kernel16p<128" in f.fmha_forward_kernel(f.CFK_FP16, 1, 40, 2048, 2048 + 64, 128)    # (a key length with a tile left over)
+    # query lengths that leave the last 256-row tile partly filled: the 8-wave shape while at most a quarter of the rows idle
+    assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 2016, 2048, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
+    assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 384, 2048, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
+    assert f.fmha_forward_kernel(f.CFK_FP16, 8, 128, 128, 2048, 128) == "fmha_fwd_kernel<128,64,4,2,0,0,0,0,1,0,0,0>"     # (half would)
+    assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 320, 2048, 128) == "fmha_fwd_kernel<128,64,4,2,0,0,0,0,1,0,0,0>"
+    assert f.fmha_forward_kernel(f.CFK_FP16, 4, 16, 160, 2048, 128) == "fmha_fwd_kernel16p<128,64,4,1,0,0,0,0,2,0,1,1>"    # (128-row tiles: no smaller one to prefer)
     assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 1, 8, 8192, 8192 + 32, 256)    # (head dim 256: whole 128s only)
     assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 16, 4096, 4096 + 64, 128)  # (e4m3: whole 256s only)
     assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 8, 4096, 4096, 128) == "fmha_fwd_kernel8p<128,64,4,2,1,1,0,0,2,0,0,1>"   # 128 items: the 4-wave shape
