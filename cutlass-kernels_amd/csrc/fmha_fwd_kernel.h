@@ -784,15 +784,15 @@ constexpr auto fmha_kernel_of() {
   else return &fmha_fwd_kernel<C>;
 }
 
-// Persistent workgroups (FmhaCfg::ASM): one per CU, a multiple of the 8 XCDs so that a workgroup's items stay on its XCD.
+// Persistent workgroups (FmhaCfg::ASM): one per CU -- a multiple of the 8 XCDs, so that a workgroup's items stay on its
+// XCD -- or one per item where there are no more items than CUs (any number: nobody takes a second item then).
 inline int persistent_grid(int n_items) {
   static const int cus = [] {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) n = 256;
     return n / 8 * 8;
   }();
-  const int g = n_items < cus ? n_items / 8 * 8 : cus;
-  return g < 8 ? n_items : g;
+  return n_items <= cus ? n_items : cus;
 }
 
 template <class C>
@@ -829,7 +829,7 @@ template <class C>
 void fill_fmha_plan(int sq, int bh, FmhaPlan *p) {
   p->block_m = C::BM;
   p->block_n = C::BN * C::SUB;
-  p->kv_multiple = C::ASM && !C::QK8 && C::D != 256 ? C::BN : C::BN * C::SUB;
+  p->kv_multiple = C::ASM && C::D != 256 ? C::BN : C::BN * C::SUB;
   p->q_multiple = q_multiple<C>;
   p->mfma = C::M16 ? 16 : 32;
   p->lds_bytes = C::LDS_BYTES;
@@ -887,9 +887,9 @@ struct CfgList {};
 // two tiles with the two-tile step)
 template <class C>
 constexpr bool fits(int sq, int skv) {
-  // (the fp16 hand-scheduled builds at head dims 64 and 128 take up to three tiles behind the last group of four outside
+  // (the hand-scheduled builds at head dims 64 and 128 take up to three tiles behind the last group of four outside
   // their loop)
-  return sq % q_multiple<C> == 0 && skv % (C::BN * (C::ASM && !C::QK8 && C::D != 256 ? 1 : C::KPRE || C::ASM ? 4 : C::SUB)) == 0 &&
+  return sq % q_multiple<C> == 0 && skv % (C::BN * (C::ASM && C::D != 256 ? 1 : C::KPRE || C::ASM ? 4 : C::SUB)) == 0 &&
          (!C::ASM || skv >= 8 * C::BN);
 }
 
@@ -917,6 +917,10 @@ constexpr bool hand_loop_pays(long long items, int skv) {
   // reads 0.0001 % at 3072 keys, 0.0003..0.0008 % at 2048, 0.03 % at 1024 (0.005 % for the max-tracking pass) -- so
   // shorter key lengths take it only by wish (CFK_FMHA_TILE=256x128/32h or 128x128/32h: +19..50 % there))
   if (skv < 3072) return false;
+  // (from 4096 keys on the lead over the compiler-scheduled builds is 7..20 %: tiles behind the last group of four, which
+  // run outside the generated loop, cost that much or more -- 8 waves, 4160 / 4224 / 4288 keys: -3 / -12 / -3 %; 4 waves: a
+  // tie; below 4096 keys the lead is larger: 3136 / 3264 keys +8 % with 8 waves, +40 % with 4)
+  if (skv >= 4096 && skv % (4 * C::BN) != 0) return false;
   if (C::BM == 128) return items <= 256;   // (the 4-wave shape: one round of 128-row items)
   if (skv < 4096) return items > 128;      // (shorter key lengths: wherever the 4-wave shape does not apply)
   const long long rounds = (items + 255) / 256;

@@ -168,7 +168,8 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 320, 2048, 128) == "fmha_fwd_kernel<128,64,4,2,0,0,0,0,1,0,0,0>"
     assert f.fmha_forward_kernel(f.CFK_FP16, 4, 16, 160, 2048, 128) == "fmha_fwd_kernel16p<128,64,4,1,0,0,0,0,2,0,1,1>"    # (128-row tiles: no smaller one to prefer)
     assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 1, 8, 8192, 8192 + 32, 256)    # (head dim 256: whole 128s only)
-    assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 16, 4096, 4096 + 64, 128)  # (e4m3: whole 256s only)
+    assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 16, 4096, 4096 + 64, 128)  # (e4m3 from 4096 keys: whole 256s only,
+    assert "kernel8p<" in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 16, 4096, 3072 + 64, 128)      #  below that also with tiles left over)
     assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 8, 4096, 4096, 128) == "fmha_fwd_kernel8p<128,64,4,2,1,1,0,0,2,0,0,1>"   # 128 items: the 4-wave shape
     assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 9, 4096, 4096, 128)      # 288 items of 128 rows, 144 of 256: neither
     assert "kernel8p<" in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 10, 4096, 4096, 128)         # 160
