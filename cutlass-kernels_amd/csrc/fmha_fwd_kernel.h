@@ -163,9 +163,12 @@ fmha_fwd_kernel(const FmhaArgs a) {
   constexpr int PS = PV8 ? BN / 64 : BN / 16;  // K-steps of O^T
   const float kTau = a.tau;                    // deferred-rescale threshold above the running max (log2 domain)
   // e4m3 P: the reference point sits this far below the row max (the weights reach up to 464 = 2^8.86).  The pass
-  // that tracks the row max keeps it 7 below; the pass that does not (see the passes below) 2 below the first tile's
-  // max, which leaves later maxima 6.9 binades = 4.7 standard deviations of N(0,1) scores (the reference's own
-  // algorithm casts weights in (0, 1], i.e. 0 below: the small weights keep two bits more than there).
+  // that tracks the row max keeps it 7 below; the pass that does not (see the passes below) takes the first tile's max
+  // itself -- that tile's weights lie in (0, 1], the range the reference's own algorithm casts all weights in -- which
+  // leaves later maxima 8.8 binades = 6.1 standard deviations of N(0,1) scores.  (An earlier build sat 2 below that max:
+  // two more bits for the smallest weights, which the output does not show -- rms error 6.806e-4 against 6.811e-4 at 4096
+  // keys -- and 6.9 binades of head-room, which one in fourteen sets of N(0,1) tensors with 128 k rows exceeded in
+  // some row, sending that row's workgroup through the second pass.)
   float p_bias = PV8 ? 7.0f : 0.0f;
   using QReg = std::conditional_t<QK8, int8v, half8>;
   using PReg = std::conditional_t<PV8, int8v, half8>;
@@ -619,7 +622,9 @@ fmha_fwd_kernel(const FmhaArgs a) {
       for (int v = 0; v < 16; ++v) oacc[db][v] = 0.f;
     m_ref = -INFINITY, m_lane = -INFINITY, l_run = 0.f, thr_raw = -INFINITY;
     l_acc = f32x4{0.f, 0.f, 0.f, 0.f};
-    p_bias = PV8 ? (TRACK ? 7.0f : 2.0f) : 0.0f;
+    // (the direct codes have no subnormals -- everything below 2^-7 becomes 0 -- so that form keeps the reference point 2
+    // below the first tile's max: a row whose first tile holds an unusually large score would lose the bulk of its keys)
+    p_bias = PV8 ? (TRACK ? 7.0f : decltype(track)::direct ? 2.0f : 0.0f) : 0.0f;
     if constexpr (C::KPRE > 0) {
       // ---- prologue: K_0, K_1, K_2, V_0 in flight; S_0, its row max, first fragments of K_1.  n_tiles % 4 == 0.
       using T = integral_constant<bool, true>;
@@ -910,7 +915,15 @@ constexpr bool fits(int sq, int skv) {
 // every item count above (576 items of 128 rows +7..10 %, 1024 and more +22..28 %).
 template <class C>
 constexpr bool hand_loop_pays(long long items, int skv) {
-  if (!C::QK8) return C::D == 256 ? skv >= 1024 : C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;
+  if (!C::QK8) {
+    if (C::D == 256) return skv >= 1024;
+    // (key tiles behind the last group of four run outside the generated loop, at three to four times a tile's time in it:
+    // worth it from 2048 keys on and while they are few -- 2112 keys +9 %, 3008 keys with three of them a tie, 704 keys with
+    // three -15 %, 1088 keys with one -9 %)
+    const int n_tiles = skv / C::BN, n_left = n_tiles & 3;
+    if (n_left != 0 && (n_tiles < 32 || n_left * 16 > n_tiles)) return false;
+    return C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;
+  }
   // (e4m3: the hand-scheduled loop sets its reference point from the first key tile, so a row's largest weight is not an
   // exact power of two as it is for a reference point that follows the running max; over few keys the rounding of that
   // weight does not average out -- the reference's error percentage, fmha_forward.cu:638-639 with its limit of 0.001 %,
@@ -938,9 +951,10 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish
     using C = decltype(c);
     if (done || !fits<C>(sq, skv)) return;
     // (a 256-row tile whose last waves lie behind the last query row idles them: worth it while the hand-scheduled loop's
-    // lead over a 128-row build -- 20..30 % for fp16, 7..9 % for e4m3 -- outweighs the idle share of the rows)
+    // lead over a 128-row build -- 20..30 % for fp16, 7..9 % for e4m3 -- outweighs the idle share of the rows: up to a
+    // quarter of them at head dim 128 (S_q=384: +6 %), an eighth at head dim 64 (S_q=640, a sixth idle: -4 %))
     const long long padded = (long long)((sq + C::BM - 1) / C::BM) * C::BM;
-    const bool tight = C::BM <= 128 || (padded - sq) * (C::QK8 ? 16 : 4) <= padded;
+    const bool tight = C::BM <= 128 || (padded - sq) * (C::QK8 ? 16 : C::D == 64 ? 8 : 4) <= padded;
     const bool by_size = C::ASM ? tight && hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
     if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : !by_size)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;

@@ -20,8 +20,8 @@ What the loop computes (same mathematics, LDS tile formats and register layouts 
 reference: src/fmha-pipeline/fmha_consumer.h:8-73, online_softmax.h:87-207, fmha_pipe_ws.h:245-296):
   for key tile t (64 keys):  S(t)^T = K(t) . Q^T ;  P(t) = e4m3(exp2(c S(t) - m)) ;  l += rowsum P(t) ;
                              O^T += V(t)^T . P(t)^T
-with the reference point m fixed by the first tile's row max (minus 2: the weights then reach up to 4 on that tile and
-have 6.9 binades left before v_cvt_pk_fp8_f32 turns them into NaN); the caller looks for a non-finite row sum afterwards
+with the reference point m fixed by the first tile's row max (the weights then reach up to 1 on that tile and
+have 8.8 binades left before v_cvt_pk_fp8_f32 turns them into NaN); the caller looks for a non-finite row sum afterwards
 and falls back to a loop that tracks the max.  S(0) is computed by the caller.
 
 Timeline.  A tile owns T = 9 MFMA places:

@@ -125,7 +125,10 @@ def test_tile_wish_is_honoured_by_the_plan_without_gpu():
     assert lds("256x128/16h") == "163840 (128, 64, 65536)"    # key length 384: fewer than eight tiles, the wish is ignored
     assert lds("256x128/16") == "131072 (256, 128, 131072)"
     assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2048, 128)[:2] == (256, 128)  # big problem: automatic choice
-    assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 1984, 128)[:2] == (256, 128)  # ... also with tiles left over behind the last four
+    assert f.fmha_forward_plan(f.CFK_FP16, 8, 16, 2048, 2112, 128)[:2] == (256, 128)  # ... also with a tile left over behind the last four
+    assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 2048, 2112, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
+    # (... from 2048 keys on and while the tiles left over are few: 31 tiles, three of them left over, stay compiler-scheduled)
+    assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 2048, 1984, 128)
     # ... on 16x16x32 MFMAs for fp16; problems with fewer work items than half the CUs (head dims 64, 128) and e4m3 stay on 32x32
     assert f.fmha_forward_mfma(f.CFK_FP16, 8, 16, 2048, 2048, 128) == 16
     assert f.fmha_forward_mfma(f.CFK_FP16, 4, 32, 4096, 4096, 64) == 16
