@@ -955,7 +955,19 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish
     // quarter of them at head dim 128 (S_q=384: +6 %), an eighth at head dim 64 (S_q=640, a sixth idle: -4 %))
     const long long padded = (long long)((sq + C::BM - 1) / C::BM) * C::BM;
     const bool tight = C::BM <= 128 || (padded - sq) * (C::QK8 ? 16 : C::D == 64 ? 8 : 4) <= padded;
-    const bool by_size = C::ASM ? tight && hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
+    // (... and the fp16 256-row builds while what they lose -- to idle rows, to key tiles behind the last group of four
+    // (each about 2.5 tile times more) and to a last round of work items that leaves CUs idle (the 128-row builds
+    // lose about half as much to theirs) -- adds up to at most a quarter: over three draws of 100 problem sizes,
+    // automatic choice against CFK_FMHA_HANDLOOP=0, every choice that lost more than the noise summed to 0.29 or more)
+    bool stacked_ok = true;
+    if (C::ASM && !C::QK8 && C::BM > 128) {
+      const long long items = bh * (padded / C::BM), rounds = (items + 255) / 256;
+      const int n_tiles = skv / C::BN, n_left = C::D == 256 ? 0 : n_tiles & 3;
+      const double idle_rows = 1.0 - (double)sq / padded, tail = 2.5 * n_left / n_tiles;
+      const double last_round = rounds > 1 ? 1.0 - (double)items / (rounds * 256) : 0.0;
+      stacked_ok = idle_rows + tail + 0.5 * last_round <= 0.25;
+    }
+    const bool by_size = C::ASM ? tight && stacked_ok && hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
     if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : !by_size)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
     if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;

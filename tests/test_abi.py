@@ -160,7 +160,11 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 1, 8192, 8192, 256)          # (at head dim 256 from 1024 keys)
     assert "kernel16p<256" in f.fmha_forward_kernel(f.CFK_FP16, 1, 2, 1024, 1024, 256)
     assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 16, 64, 512, 512, 256)
-    assert "kernel16p<128" in f.fmha_forward_kernel(f.CFK_FP16, 1, 40, 2048, 2048 + 64, 128)    # (a key length with a tile left over)
+    assert "kernel16p<128" in f.fmha_forward_kernel(f.CFK_FP16, 1, 64, 2048, 2048 + 64, 128)    # (a key length with a tile left over)
+    # (... while idle rows, leftover tiles and a thinly filled last round of items do not add up: 320 items in two rounds
+    # and a leftover tile on top stay compiler-scheduled)
+    assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 1, 40, 2048, 2048 + 64, 128)
+    assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 8, 17, 896, 3520, 64)
     # query lengths that leave the last 256-row tile partly filled: the 8-wave shape while at most a quarter of the rows idle
     assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 2016, 2048, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
     assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 384, 2048, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
