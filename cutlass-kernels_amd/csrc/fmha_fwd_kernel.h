@@ -918,10 +918,10 @@ constexpr bool hand_loop_pays(long long items, int skv) {
   if (!C::QK8) {
     if (C::D == 256) return skv >= 1024;
     // (key tiles behind the last group of four run outside the generated loop, at three to four times a tile's time in it:
-    // worth it from 2048 keys on and while they are few -- 2112 keys +9 %, 3008 keys with three of them a tie, 704 keys with
-    // three -15 %, 1088 keys with one -9 %)
+    // worth it from 2048 keys on and while they are few -- 2112 keys +9 %, 3008 keys with three of them 0..+27 %, 704 keys
+    // with three -15 %, 1088 keys with one -9 %)
     const int n_tiles = skv / C::BN, n_left = n_tiles & 3;
-    if (n_left != 0 && (n_tiles < 32 || n_left * 16 > n_tiles)) return false;
+    if (n_left != 0 && (n_tiles < 32 || n_left * 10 > n_tiles)) return false;
     return C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;
   }
   // (e4m3: the hand-scheduled loop sets its reference point from the first key tile, so a row's largest weight is not an
@@ -951,21 +951,31 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish
     using C = decltype(c);
     if (done || !fits<C>(sq, skv)) return;
     // (a 256-row tile whose last waves lie behind the last query row idles them: worth it while the hand-scheduled loop's
-    // lead over a 128-row build -- 20..30 % for fp16, 7..9 % for e4m3 -- outweighs the idle share of the rows: up to a
-    // quarter of them at head dim 128 (S_q=384: +6 %), an eighth at head dim 64 (S_q=640, a sixth idle: -4 %))
+    // lead over a 128-row build -- 20..30 % for fp16, 7..9 % for e4m3 from 4096 keys on and more below -- outweighs the
+    // idle share of the rows: up to a quarter of them at head dim 128 (S_q=384: +6 %), an eighth at head dim 64 (S_q=640,
+    // a sixth idle: -4 %) and for e4m3 below 4096 keys (S_q=1664, 3712 keys: +12 %), a sixteenth for e4m3 above)
     const long long padded = (long long)((sq + C::BM - 1) / C::BM) * C::BM;
-    const bool tight = C::BM <= 128 || (padded - sq) * (C::QK8 ? 16 : C::D == 64 ? 8 : 4) <= padded;
+    const bool tight = C::BM <= 128 || (padded - sq) * (C::QK8 ? (skv < 4096 ? 8 : 16) : C::D == 64 ? 8 : 4) <= padded;
     // (... and the fp16 256-row builds while what they lose -- to idle rows, to key tiles behind the last group of four
     // (each about 2.5 tile times more) and to a last round of work items that leaves CUs idle (the 128-row builds
     // lose about half as much to theirs) -- adds up to at most a quarter: over three draws of 100 problem sizes,
     // automatic choice against CFK_FMHA_HANDLOOP=0, every choice that lost more than the noise summed to 0.29 or more)
     bool stacked_ok = true;
+    if (C::ASM && C::QK8 && C::BM > 128 && skv < 4096) {
+      // (e4m3 below 4096 keys, where no rule on the last round applies: idle rows count double -- S_q=896 in 256-row tiles with
+      // 528 items in three rounds -12 %; S_q=1664 with 1015 items +12 %; whole tiles with 288 items in two rounds +8 %)
+      const long long items = bh * (padded / C::BM), rounds = (items + 255) / 256;
+      const double last_round = rounds > 1 ? 1.0 - (double)items / (rounds * 256) : 0.0;
+      stacked_ok = 2.0 * (1.0 - (double)sq / padded) + 0.5 * last_round <= 0.25;
+    }
     if (C::ASM && !C::QK8 && C::BM > 128) {
       const long long items = bh * (padded / C::BM), rounds = (items + 255) / 256;
       const int n_tiles = skv / C::BN, n_left = C::D == 256 ? 0 : n_tiles & 3;
       const double idle_rows = 1.0 - (double)sq / padded, tail = 2.5 * n_left / n_tiles;
       const double last_round = rounds > 1 ? 1.0 - (double)items / (rounds * 256) : 0.0;
-      stacked_ok = idle_rows + tail + 0.5 * last_round <= 0.25;
+      // (head dim 64: the larger lead; below 1024 keys, where the loop is all head and tail and the lead a few per cent, a
+      // thin last round counts in full: 512 keys, 310 items -16 %)
+      stacked_ok = n_tiles < 16 ? idle_rows + last_round <= 0.2 : idle_rows + tail + 0.5 * last_round <= (C::D == 64 ? 0.32 : 0.25);
     }
     const bool by_size = C::ASM ? tight && stacked_ok && hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
     if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : !by_size)) return;
