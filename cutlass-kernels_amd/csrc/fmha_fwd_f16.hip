@@ -60,7 +60,7 @@ bool dispatch(int head_dim, int sq, int skv, int bh, bool tap_s, F &&f) {
   }
   switch (head_dim) {
     case 64: select_tile<All64, CfgList<K64_32x64, A64_256x128, A64_128x128, N64_128x64, C64_128x64>, C64_128x64>(sq, skv, bh, f); return true;
-    case 128: select_tile<All128, CfgList<K128_32x64, A128_256x128, A128_128x128, N128_256x128, N128_256x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
+    case 128: select_tile<All128, CfgList<K128_32x64, A128_256x128, A128_128x128, N128_256x128, N128_256x64, N128_128x64, C128_256x64P, C128_256x64, C128_128x64>, C128_128x64>(sq, skv, bh, f); return true;
     default: return false;
   }
 }

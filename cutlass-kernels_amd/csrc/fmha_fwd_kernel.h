@@ -940,6 +940,9 @@ constexpr bool hand_loop_pays(long long items, int skv) {
   return items >= 160 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
 }
 
+// (The compiler-scheduled fp16 256-row builds need key length to pay: B=8 H=27 S_q=1536 D=128 with 896 keys 723 TFLOP/s on
+// 256 x 128 keys, 871 on 256 x 64, 947 on 128 x 64, all on 16x16x32 MFMAs; with 1536 keys 1036 / 1038 / 1014.  e4m3, B=8 H=32
+// S_q=2048 D=128: 1024 keys 1445 on 256 x 128 against 1517 on 128 x 64, 1536 keys 1529 / 1573, 2048 keys 1702 / 1705.)
 // Calls f with the first instantiation of the list that fits the shape and the wish.  Without a wish for the query
 // rows, the hand-scheduled builds are taken where they pay (above), other tiles above 128 rows and the other 16x16x32
 // builds (slower where launch and prologue dominate) only for big problems (size 2: enough workgroups to fill 256 CUs
@@ -977,7 +980,8 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish
       // thin last round counts in full: 512 keys, 310 items -16 %)
       stacked_ok = n_tiles < 16 ? idle_rows + last_round <= 0.2 : idle_rows + tail + 0.5 * last_round <= (C::D == 64 ? 0.32 : 0.25);
     }
-    const bool by_size = C::ASM ? tight && stacked_ok && hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv) : !((C::BM > 128 || C::M16) && size != 2);
+    const bool by_size = C::ASM ? tight && stacked_ok && hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv)
+                                : !((C::BM > 128 || C::M16) && size != 2) && !(C::BM > 128 && skv < (C::PV8 ? 2048 : C::QK8 ? 0 : 1152));
     if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : !by_size)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
     if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;

@@ -165,6 +165,12 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     # and a leftover tile on top stay compiler-scheduled)
     assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 1, 40, 2048, 2048 + 64, 128)
     assert "kernel16p<" not in f.fmha_forward_kernel(f.CFK_FP16, 8, 17, 896, 3520, 64)
+    # big problems with short keys: the compiler-scheduled 256-row builds need key length to pay (fp16 below 1152 keys and
+    # e4m3 below 2048 take 128-row tiles)
+    assert f.fmha_forward_kernel(f.CFK_FP16, 8, 27, 1536, 896, 128) == "fmha_fwd_kernel16<128,64,4,2,0,0,0,0,1,0,1,0>"
+    assert f.fmha_forward_kernel(f.CFK_FP16, 8, 32, 2048, 1216, 128) == "fmha_fwd_kernel16<128,64,8,2,0,0,0,0,1,0,1,0>"
+    assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 8, 32, 2048, 1024, 128) == "fmha_fwd_kernel<128,64,4,2,1,1,0,0,1,0,0,0>"
+    assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 8, 32, 2048, 2048, 128) == "fmha_fwd_kernel<128,64,8,2,1,1,0,0,2,0,0,0>"
     # query lengths that leave the last 256-row tile partly filled: the 8-wave shape while at most a quarter of the rows idle
     assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 2016, 2048, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
     assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 384, 2048, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
