@@ -33,9 +33,9 @@ TRAFFIC_SOURCE = {
     "cfg2": dict(profile="profiles/fmha_fwd_f16_B8_H16_S2048_D128.md", kernel="fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>",
                  fetch_kib=107998, write_kib=65536),
     "cfg3": dict(profile="profiles/fmha_fwd_f16_B2_H8_S8192_D256.md", kernel="fmha_fwd_kernel16p<256,32,4,1,0,0,0,0,2,0,1,1>",
-                 fetch_kib=172631, write_kib=65536),
+                 fetch_kib=172627, write_kib=65536),
     "cfg4": dict(profile="profiles/fmha_fwd_fp8_B4_H16_S4096_D128.md", kernel="fmha_fwd_kernel8p<128,64,8,2,1,1,0,0,2,0,0,1>",
-                 fetch_kib=53708, write_kib=65536),
+                 fetch_kib=53713, write_kib=65536),
     "cfg5": dict(profile="profiles/gemm_M8192_N8192_K8192.md", kernel="gemm_kernel16<0,4>", fetch_kib=787716, write_kib=131072),
 }
 
