@@ -46,7 +46,8 @@ CASES = {
                     "f16ntclimb:1,512,2,128,576", "f16ntclimb:1,512,2,64,704",    # (the spike key inside the loop's tiles, and behind them)
                     # ... a last query tile filled to a whole number of waves: 2x16 heads x 2016 rows, 3x16x2016 (second items)
                     "f16nt:2,416,3,128,768", "f16nt:2,2016,16,128,2048", "f16nt:3,2016,16,64,2112", "f16ntclimb:2,288,2,128,768",
-                    "f16ntclimb:2,352,2,64,640", "f16:2,416,2,128,768"],
+                    "f16ntclimb:2,352,2,64,640", "f16:2,416,2,128,768",
+                    "f16ntclimb:2,352,2,64,2112", "f16nt:3,2016,16,128,2240", "f16ntclimb:2,288,2,128,2176"],   # (... with leftover key tiles as well)
     # ... and its head-dim-256 shape (4 waves, one per SIMD, 32-key tiles; key length a multiple of 128, at least 256):
     # 3x6 heads x 2048 rows = 288 items of 128 rows (32 workgroups take a second one), climbing keys, taps
     "128x64/16h": ["f16nt:1,256,2,256", "f16nt:1,128,3,256,640", "f16nt:3,2048,6,256,512", "f16ntclimb:1,256,2,256,512",
@@ -68,12 +69,14 @@ CASES = {
     # fewer tiles than waves, with tiles left over, query lengths that no other tile divides, taps, climbing keys
     "32x64": ["f16:1,512,8,64", "f16:1,512,2,128", "f16:2,96,3,64,64", "f16:1,160,2,128,192", "f16:1,128,2,64,1216", "f16nt:1,256,2,128,640",
               "f16climb:1,256,2,64,512", "f16climb:1,128,2,128,1024", "f16:3,2048,4,128,2048"],
-    "256x128/32h": ["f8:1,512,2,128,4160", "f8:2,512,3,128,4288", "f8climb:1,256,2,128,4224", "f8:3,4096,10,128,3136",   # (one to three tiles behind the last group of four)
+    "256x128/32h": ["f8climb:2,288,2,128,3264", "f8:2,1184,3,128,3136",   # (leftover key tiles and a partly filled last query tile together)
+                    "f8:1,512,2,128,4160", "f8:2,512,3,128,4288", "f8climb:1,256,2,128,4224", "f8:3,4096,10,128,3136",   # (one to three tiles behind the last group of four)
                     "f8:1,512,2,128,512", "f8:2,512,2,128,1280", "f8:1,512,2,128,3072", "f8climb:1,256,2,128,768",   # (key lengths below 3072:
                     "f8:2,1184,2,128,4096", "f8:2,4064,10,128,4096", "f8climb:2,288,2,128,4096",   # (partly filled last query tile)
                     "f8:1,256,2,128,4096", "f8:1,512,1,128,4352", "f8:2,4096,10,128", "f8climb:1,256,2,128,4096", "f8climb:5,1024,13,128,4096"],
     # ... and its 4-wave shape (128 query rows, two copies per wave and tile): 1x9 heads x 4096 rows = 288 items
-    "128x128/32h": ["f8:1,256,2,128,4160", "f8:2,384,3,128,3264", "f8climb:1,128,2,128,4288", "f8:1,4096,9,128,3136",     # (likewise)
+    "128x128/32h": ["f8climb:2,224,2,128,3264", "f8:2,1184,3,128,3136",   # (likewise)
+                    "f8:1,256,2,128,4160", "f8:2,384,3,128,3264", "f8climb:1,128,2,128,4288", "f8:1,4096,9,128,3136",     # (likewise)
                     "f8:1,256,2,128,512", "f8:1,384,3,128,3072", "f8climb:1,128,2,128,1024",   #  by wish only)
                     "f8:2,1184,2,128,4096", "f8:1,4064,9,128,4096", "f8climb:2,224,2,128,4096",    # (partly filled last query tile)
                     "f8:1,128,2,128,4096", "f8:1,256,1,128,4352", "f8:1,4096,9,128", "f8climb:1,128,2,128,4096", "f8climb:5,512,13,128,4096"],
