@@ -154,12 +154,13 @@ int cfk_fmha_forward(const cfk_fmha_fwd_params *p, void *stream) {
   // weight (<= 6 %) averages out over long key sequences but shows in the reference's error-percentage measure on short
   // ones, so those run with tau = 0.
   a.tau = p->v_dtype != CFK_FP8_E4M3 ? 8.0f : p->seqlen_kv < 2048 ? 0.0f : 1.0f;
-  // e4m3 P: the pass without a row max per tile keeps the small weights of a row less well (its reference point sits
-  // 2, not 7, below a max, and only the first tile's).  Over the 4096 keys of the reference's own problem that is far
-  // inside its error-percentage gate (fmha_forward.cu:638-639: 0.0000 % against 0.001 %); at 2048 keys the same measure
-  // reads 0.0011 % for head dim 64, so key lengths below 4096 take the max-tracking pass only.
+  // e4m3 P: in the pass without a row max per tile the reference point comes from the first tile, so a row's largest
+  // weight is not the exact power of two it is under a running max, and over few keys the rounding of that weight shows in
+  // the reference's error-percentage gate (fmha_forward.cu:638-639, limit 0.001 %): 0.0000 % over the 4096 keys of the
+  // reference's own problem, 0.00001..0.00006 % at 3072 and 3584 keys, 0.0001..0.0003 % at 2560, 0.0005..0.0013 % at 2048
+  // (head dims 128, 256, 64).  Key lengths below 3072 take the max-tracking pass only.
   a.direct_p = g_fast_e4m3.load(std::memory_order_relaxed);
-  a.track_only = cfk::predictable_latency() || (p->v_dtype == CFK_FP8_E4M3 && p->seqlen_kv < 4096) ? 1 : 0;
+  a.track_only = cfk::predictable_latency() || (p->v_dtype == CFK_FP8_E4M3 && p->seqlen_kv < 3072) ? 1 : 0;
   hipError_t e;
   a.s_scale = p->dtype == CFK_FP16 ? p->softmax_scale : p->softmax_scale * p->q_descale * p->k_descale;
   if (p->dtype == CFK_FP16) {

@@ -910,9 +910,9 @@ constexpr bool fits(int sq, int skv) {
 // e4m3: the 8-wave shape from 160 items on (+8..13 %; at 128 items -11 %) and only while the last round of items keeps
 // four fifths of the workgroups busy (320 items -8 %, 384 items -5 %: the 128-row tile has twice the workgroups to even
 // out the tail); up to 256 items of 128 rows the 4-wave shape (+9..20 % over the compiler-scheduled 128-row build).
-// Those are the figures from 4096 keys on.  At 512 to 3072 keys the compiler-scheduled e4m3 builds lose more to their
-// prologue and epilogue: there the 4-wave shape is +19..50 % up to 256 items of 128 rows and the 8-wave shape +7..38 % at
-// every item count above (576 items of 128 rows +7..10 %, 1024 and more +22..28 %).
+// Those figures hold from 3072 keys on, where every e4m3 build starts with the pass that takes no row max per tile (3072
+// keys: 4 waves +10..16 %; 8 waves +6..12 % at 288 to 480 items of 128 rows and 896 to 960, -3..-8 % at 576 to 768).  Below,
+// the compiler-scheduled builds run their max-tracking pass only and are 19..50 % slower than this loop.
 template <class C>
 constexpr bool hand_loop_pays(long long items, int skv) {
   if (!C::QK8) {
@@ -924,18 +924,16 @@ constexpr bool hand_loop_pays(long long items, int skv) {
     if (n_left != 0 && (n_tiles < 32 || n_left * 10 > n_tiles)) return false;
     return C::BM == 128 ? items <= 256 && skv >= 1024 : items > 128;
   }
-  // (e4m3: the hand-scheduled loop sets its reference point from the first key tile, so a row's largest weight is not an
-  // exact power of two as it is for a reference point that follows the running max; over few keys the rounding of that
-  // weight does not average out -- the reference's error percentage, fmha_forward.cu:638-639 with its limit of 0.001 %,
-  // reads 0.0001 % at 3072 keys, 0.0003..0.0008 % at 2048, 0.03 % at 1024 (0.005 % for the max-tracking pass) -- so
-  // shorter key lengths take it only by wish (CFK_FMHA_TILE=256x128/32h or 128x128/32h: +19..50 % there))
+  // (e4m3: the first pass sets its reference point from the first key tile, so a row's largest weight is not an exact
+  // power of two as it is for a reference point that follows the running max; over few keys the rounding of that weight
+  // does not average out -- cfk_api.hip has the figures -- so key lengths below 3072 take the max-tracking pass, which this
+  // build only has as an unpipelined fall-back: there it runs by wish only (CFK_FMHA_TILE=256x128/32h or 128x128/32h;
+  // 19..50 % faster than the max-tracking compiler-scheduled builds))
   if (skv < 3072) return false;
-  // (from 4096 keys on the lead over the compiler-scheduled builds is 7..20 %: tiles behind the last group of four, which
-  // run outside the generated loop, cost that much or more -- 8 waves, 4160 / 4224 / 4288 keys: -3 / -12 / -3 %; 4 waves: a
-  // tie; below 4096 keys the lead is larger: 3136 / 3264 keys +8 % with 8 waves, +40 % with 4)
+  // (tiles behind the last group of four, which run outside the generated loop, cost about what the loop gains: 3136
+  // keys +4..6 %, 4160 / 4224 / 4288 keys -3 / -12 / -3 % with 8 waves and a tie with 4: taken below 4096 keys only)
   if (skv >= 4096 && skv % (4 * C::BN) != 0) return false;
   if (C::BM == 128) return items <= 256;   // (the 4-wave shape: one round of 128-row items)
-  if (skv < 4096) return items > 128;      // (shorter key lengths: wherever the 4-wave shape does not apply)
   const long long rounds = (items + 255) / 256;
   return items >= 160 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
 }
@@ -954,23 +952,16 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish
     using C = decltype(c);
     if (done || !fits<C>(sq, skv)) return;
     // (a 256-row tile whose last waves lie behind the last query row idles them: worth it while the hand-scheduled loop's
-    // lead over a 128-row build -- 20..30 % for fp16, 7..9 % for e4m3 from 4096 keys on and more below -- outweighs the
-    // idle share of the rows: up to a quarter of them at head dim 128 (S_q=384: +6 %), an eighth at head dim 64 (S_q=640,
-    // a sixth idle: -4 %) and for e4m3 below 4096 keys (S_q=1664, 3712 keys: +12 %), a sixteenth for e4m3 above)
+    // lead over a 128-row build -- 20..30 % for fp16, 7..9 % for e4m3 -- outweighs the idle share of the rows: up to a
+    // quarter of them at head dim 128 (S_q=384: +6 %), an eighth at head dim 64 (S_q=640, a sixth idle: -4 %), a
+    // sixteenth for e4m3)
     const long long padded = (long long)((sq + C::BM - 1) / C::BM) * C::BM;
-    const bool tight = C::BM <= 128 || (padded - sq) * (C::QK8 ? (skv < 4096 ? 8 : 16) : C::D == 64 ? 8 : 4) <= padded;
+    const bool tight = C::BM <= 128 || (padded - sq) * (C::QK8 ? 16 : C::D == 64 ? 8 : 4) <= padded;
     // (... and the fp16 256-row builds while what they lose -- to idle rows, to key tiles behind the last group of four
     // (each about 2.5 tile times more) and to a last round of work items that leaves CUs idle (the 128-row builds
     // lose about half as much to theirs) -- adds up to at most a quarter: over three draws of 100 problem sizes,
     // automatic choice against CFK_FMHA_HANDLOOP=0, every choice that lost more than the noise summed to 0.29 or more)
     bool stacked_ok = true;
-    if (C::ASM && C::QK8 && C::BM > 128 && skv < 4096) {
-      // (e4m3 below 4096 keys, where no rule on the last round applies: idle rows count double -- S_q=896 in 256-row tiles with
-      // 528 items in three rounds -12 %; S_q=1664 with 1015 items +12 %; whole tiles with 288 items in two rounds +8 %)
-      const long long items = bh * (padded / C::BM), rounds = (items + 255) / 256;
-      const double last_round = rounds > 1 ? 1.0 - (double)items / (rounds * 256) : 0.0;
-      stacked_ok = 2.0 * (1.0 - (double)sq / padded) + 0.5 * last_round <= 0.25;
-    }
     if (C::ASM && !C::QK8 && C::BM > 128) {
       const long long items = bh * (padded / C::BM), rounds = (items + 255) / 256;
       const int n_tiles = skv / C::BN, n_left = C::D == 256 ? 0 : n_tiles & 3;

@@ -156,8 +156,7 @@ int cfk_gemm(const cfk_gemm_params *p, void *stream);
 typedef enum cfk_option {
   /* 1: no optimistic first pass.  Two kernels first walk the keys with a softmax reference point fixed by the first key
    * tile (no row max per tile) and, only if some weight left the range of P's type, walk them again tracking the running
-   * max as the reference does on every tile (online_softmax.h:123-165): e4m3 P from 4096 keys on (3072 for the
-   * hand-scheduled head-dim-128 kernel), and fp16 problems
+   * max as the reference does on every tile (online_softmax.h:123-165): e4m3 P from 3072 keys on, and fp16 problems
    * with more work items than half the CUs.  On scores that climb along the key axis that costs up to twice the time.  With this option
    * every call takes the max-tracking path from the start: the same results to rounding, a run time that does not
    * depend on the data (a few per cent slower on ordinary data).  0 (default): two passes where they pay. */

@@ -71,7 +71,7 @@ def _load_dump(d):
                                              (1, 128, ["seq=1088"]), (1, 256, ["seq=608"]), (2, 128, ["seq=4160"])])
 def test_driver_reference_check_and_dump(tmp_path, prec, head, extra):
     # fp8 needs the reference's own sequence length for its percentage criterion; fp16 passes at any length
-    seq = 4096 if prec == 2 else 512   # (e4m3 P: the two-pass path starts at 4096 keys)
+    seq = 4096 if prec == 2 else 512   # (e4m3 P: the two-pass path starts at 3072 keys)
     seq = next((int(e[4:]) for e in extra if e.startswith("seq=")), seq)
     extra = [e for e in extra if not e.startswith("seq=")]
     out = _run(f"--prec-type={prec}", "--batch-size=2", f"--dim-size={2 * head}", f"--head-size={head}",

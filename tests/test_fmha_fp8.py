@@ -84,7 +84,7 @@ def test_shortest_and_odd_key_tile_counts(B, S, H, D, Skv):
                                          (2, 2048, 32, 128, 2048)])
 def test_scores_that_climb_along_the_keys_move_the_reference_point(mode, B, S, H, D, Skv):
     # the deferred rescale's slow path, many times per row (e4m3 P has two binades of head-room above the row max of
-    # the moment, so here almost every tile takes it); from 4096 keys on the e4m3 kernel starts in its pass without a row
+    # the moment, so here almost every tile takes it); from 3072 keys on the e4m3 kernel starts in its pass without a row
     # max per tile, finds non-finite rows and walks the keys again (the tests of the second pass below).  The last shape is large enough for the automatic
     # choice of the 256-row tile (two sub-tiles per barrier for e4m3 P).
     import torch
@@ -345,7 +345,7 @@ def test_config4_subset_check():
     assert not np.any(np.isnan(got))
 
 
-# ---- the two-pass e4m3 kernel (from 4096 keys on): first pass without a row max per tile, second pass only where a
+# ---- the two-pass e4m3 kernel (from 3072 keys on): first pass without a row max per tile, second pass only where a
 # weight left the range of e4m3.  Every instantiation that can take the second pass is driven through it here.
 def _climb_case(B, S, H, D, Skv, v_layout=None, ramp=4.0, spike=8.0):
     import torch
@@ -407,10 +407,10 @@ def test_second_pass_for_a_single_row(D, where):
 
 def test_both_sides_of_the_key_length_where_the_passes_change():
     # below 2048 keys: one pass whose reference point follows the running max (tau = 0); from 2048 on it moves only when it
-    # must (deferred rescale); from 4096 on: two passes.  The same operands, cut on both sides of each boundary.
+    # must (deferred rescale); from 3072 on: two passes.  The same operands, cut on both sides of each boundary.
     B, S, H, D = 1, 256, 2, 128
     q, k, v = pkg.testbed.qkv(B, S, H, D, seqlen_kv=4096)
-    for skv in (1984, 2048, 4032, 4096):
+    for skv in (1984, 2048, 3008, 3072, 4096):
         got, (qf, kf, vf) = _run(q, k[:, :skv], v[:, :skv])
         ref = oracle.attention_f32(qf, kf, vf)["O"]
         err, (ok, pct) = max_abs(got, ref), oracle.verify_tensor(got, ref, ERRPCT_FP8)

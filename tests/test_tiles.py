@@ -15,6 +15,8 @@ CASES = {
     "128x64": ["f16:1,512,2,64", "f16:1,512,2,128", "f16climb:1,256,2,128,384", "f8:1,2048,2,64", "f8:1,2048,2,128", "f8:1,2048,1,256",
                "f8climb:1,256,2,64,4096", "f8climb:1,256,2,128,4096", "f8climb:1,128,1,256,4096", "f8:1,4096,1,64", "f8:1,4096,1,128", "f8:1,4096,1,256",
                "hyb:1,512,2,64", "hyb:1,512,2,128", "f16:1,256,2,256", "f16climb:1,256,1,256,192",
+               # ... 3072 keys, where the pass without a row max per tile starts
+               "f8:1,3072,2,64", "f8:1,3072,1,128", "f8:1,3072,1,256", "f8climb:1,256,2,64,3072", "f8climb:1,256,2,128,3072", "f8climb:1,128,1,256,3072",
                # ... a last query tile filled to a whole number of waves (32 rows each)
                "f16:2,160,2,64,192", "f16:2,288,3,128,192", "f16:2,160,2,256,128", "f16climb:2,160,2,128,384", "f8:2,160,2,64,2048",
                "f8:2,288,2,128,2048", "f8:2,96,1,256,2048", "f8climb:2,160,2,128,4096", "hyb:2,160,2,64,512", "hyb:2,96,2,128,512"],
@@ -23,7 +25,7 @@ CASES = {
                "f8climb:1,256,2,128,4096", "f8:1,4096,1,128"],
     "128x128": ["f16:2,224,2,64,256", "f8:2,160,2,64,2048", "hyb:2,160,2,64,512", "f16:1,512,2,64", "f16:1,512,2,128", "f16:1,384,2,128", "f8:1,2048,2,64", "f8:1,2048,2,128",
                 "f8:1,2048,1,256", "hyb:1,512,2,64", "f8climb:1,256,2,64,4096", "f8climb:1,256,2,128,4096", "f8climb:1,128,1,256,4096", "f8:1,4096,1,64", "f8:1,4096,1,128"],
-    "256x128": ["f16:2,416,2,128,384", "f8:2,1184,2,128,2048", "f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128,384", "f8:1,2048,2,128", "hyb:1,512,2,128", "f8climb:1,256,2,128,4096", "f8:1,4096,1,128"],
+    "256x128": ["f8:1,3072,1,128", "f8climb:1,256,2,128,3072", "f16:2,416,2,128,384", "f8:2,1184,2,128,2048", "f16:1,512,2,64", "f16:1,512,2,128", "f16:1,768,2,128,384", "f8:1,2048,2,128", "hyb:1,512,2,128", "f8climb:1,256,2,128,4096", "f8:1,4096,1,128"],
     "128x32": ["f16:1,256,2,256", "hyb:1,256,2,256", "f16:2,96,2,256,256", "hyb:2,224,2,256,256"],
     # the fp16 builds on 16x16x32 MFMAs
     "128x64/16": ["f16:1,512,2,64", "f16:1,512,2,128", "f16:2,384,3,128,192", "f16:1,256,2,64,64", "f16climb:1,256,2,64,512",
@@ -62,7 +64,7 @@ CASES = {
                     "f16:1,256,2,64,512", "f16climb:1,256,2,64,1024",
                     "f16nt:1,256,2,128,1088", "f16nt:1,2048,20,128,1216", "f16nt:1,256,2,64,1216", "f16ntclimb:1,256,2,64,1088", "f16ntclimb:1,128,2,128,576",
                     "f16nt:2,160,3,128,1088", "f16nt:1,2016,20,64,1216", "f16ntclimb:2,224,2,128,768", "f16:2,96,2,64,512"],   # (partly filled last tile)
-    # the e4m3 build with the hand-scheduled loop and persistent workgroups (key length a multiple of 256, from 4096): the
+    # the e4m3 build with the hand-scheduled loop and persistent workgroups (by the automatic choice from 3072 keys): the
     # scheduled loop, 4352 keys (an odd number of loop turns), 2x10 heads x 4096 rows = 320 items (a quarter of the
     # workgroups take a second one), climbing keys (the vote, the max-tracking loop, then a next item: 5x13x1024 rows = 260)
     # 32 query rows per workgroup, the eight waves split the keys (the automatic choice for small grids): key lengths with
