@@ -43,7 +43,9 @@ fi
 if [[ ${1:-fp8} == fp8 ]]; then
   sweep "--prec-type=2 --gemm2-fp8=true" 128 4096 "256x128/32h 128x128/32h" 2 4 6 8 10 12 16 20 24 28 32 64
   sweep "--prec-type=2 --gemm2-fp8=true" 128 16384 "256x128/32h 128x128/32h" 1 2 4
-  sweep "--prec-type=2 --gemm2-fp8=true" 128 3072 "256x128/32h 128x128/32h" 4 8 12 16 24 28 32 40
+  sweep "--prec-type=2 --gemm2-fp8=true" 128 3072 "256x128/32h 128x128/32h" 4 8 12 16 20 24 28 32 40 64
+  sweep "--prec-type=2 --gemm2-fp8=true" 128 3136 "256x128/32h 128x128/32h" 8 16 32
+  sweep "--prec-type=2 --gemm2-fp8=true" 128 3584 "256x128/32h 128x128/32h" 8 20 32
   # (below 3072 keys the automatic choice stays off the hand-scheduled e4m3 builds for accuracy, not for speed)
   sweep "--prec-type=2 --gemm2-fp8=true" 128 2048 "256x128/32h 128x128/32h" 8 16 20 32 64
   sweep "--prec-type=2 --gemm2-fp8=true" 128 1024 "256x128/32h 128x128/32h" 16 32 64 128
