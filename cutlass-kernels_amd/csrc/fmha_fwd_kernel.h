@@ -907,7 +907,7 @@ constexpr bool fits(int sq, int skv) {
 // +9 %; at 128 items a tie, at 96 -4 %: there the 128-row tile's twice as many workgroups count).  Up to 256 items of 128
 // rows -- one round -- those head dims take the same loops in their 4-wave shape (128 rows, one wave per SIMD): +11..20 %
 // over the compiler-scheduled 128-row builds from 1024 keys on (2048 keys +12 %, 8192 +20 %, 1024 +2..6 %, 512 -5 %).
-// e4m3: the 8-wave shape from 160 items on (+8..13 %; at 128 items -11 %) and only while the last round of items keeps
+// e4m3: the 8-wave shape from more than 128 items on (132 to 156 items +7..11 %, 160 and more +8..13 %; at 128 items -11 %) and only while the last round of items keeps
 // four fifths of the workgroups busy (320 items -8 %, 384 items -5 %: the 128-row tile has twice the workgroups to even
 // out the tail); up to 256 items of 128 rows the 4-wave shape (+9..20 % over the compiler-scheduled 128-row build).
 // Those figures hold from 3072 keys on, where every e4m3 build starts with the pass that takes no row max per tile (3072
@@ -935,7 +935,7 @@ constexpr bool hand_loop_pays(long long items, int skv) {
   if (skv >= 4096 && skv % (4 * C::BN) != 0) return false;
   if (C::BM == 128) return items <= 256;   // (the 4-wave shape: one round of 128-row items)
   const long long rounds = (items + 255) / 256;
-  return items >= 160 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
+  return items > 128 && (rounds == 1 || items * 5 >= rounds * 256 * 4);
 }
 
 // (The compiler-scheduled fp16 256-row builds need key length to pay: B=8 H=27 S_q=1536 D=128 with 896 keys 723 TFLOP/s on

@@ -147,7 +147,7 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     finally:
         f.set_option(f.CFK_OPT_PREDICTABLE_LATENCY, 0)
     # where the hand-scheduled persistent builds start (one workgroup per CU): fp16 from more 256-row items than half the
-    # CUs (head dim 256, 128-row items on either side: always); e4m3 from 160 items, while the last round keeps four
+    # CUs (head dim 256, 128-row items on either side: always); e4m3 likewise, while the last round keeps four
     # fifths of the CUs busy
     assert f.fmha_forward_kernel(f.CFK_FP16, 1, 16, 2048, 2048, 128) == "fmha_fwd_kernel16p<128,64,4,1,0,0,0,0,2,0,1,1>"   # 128 items: the 4-wave shape
     assert f.fmha_forward_kernel(f.CFK_FP16, 1, 6, 2048, 2048, 64) == "fmha_fwd_kernel16p<64,64,4,1,0,0,0,0,2,0,1,1>"     # (up to 256 items of 128 rows,
@@ -181,7 +181,7 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 16, 4096, 4096 + 64, 128)  # (e4m3 from 4096 keys: whole 256s only,
     assert "kernel8p<" in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 16, 4096, 3072 + 64, 128)      #  below that also with tiles left over)
     assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 8, 4096, 4096, 128) == "fmha_fwd_kernel8p<128,64,4,2,1,1,0,0,2,0,0,1>"   # 128 items: the 4-wave shape
-    assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 9, 4096, 4096, 128)      # 288 items of 128 rows, 144 of 256: neither
+    assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 9, 4096, 4096, 128) == "fmha_fwd_kernel8p<128,64,8,2,1,1,0,0,2,0,0,1>"   # 288 items of 128 rows, 144 of 256
     assert "kernel8p<" in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 10, 4096, 4096, 128)         # 160
     assert "kernel8p<" in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 16, 4096, 4096, 128)         # 256: one round
     assert "kernel8p<" not in f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, 20, 4096, 4096, 128)     # 320: a quarter-full second round
