@@ -971,8 +971,14 @@ bool first_fit(CfgList<Cs...>, int sq, int skv, long long bh, int size, TileWish
       // thin last round counts in full: 512 keys, 310 items -16 %)
       stacked_ok = n_tiles < 16 ? idle_rows + last_round <= 0.2 : idle_rows + tail + 0.5 * last_round <= (C::D == 64 ? 0.32 : 0.25);
     }
+    // (the compiler-scheduled 256-row builds for e4m3 Q and K -- one 8-wave workgroup per CU -- against the 128-row tile, at
+    // 2048 and 4096 keys: 128 items of 256 rows -20 %, 160 to 256 +2..8 %, 320 and 384 -7..-13 %, 512 +1..5 %, 576 -7..-10 %,
+    // 768 0..+4 %: taken while their rounds of 256 workgroups fill)
+    const long long items256 = bh * ((sq + 255) / 256), rounds256 = (items256 + 255) / 256;
+    const bool fills256 = sq % 256 == 0 && items256 >= 160 && (rounds256 == 1 || items256 * 5 >= rounds256 * 256 * 4);
     const bool by_size = C::ASM ? tight && stacked_ok && hand_loop_pays<C>(bh * ((sq + C::BM - 1) / C::BM), skv)
-                                : !((C::BM > 128 || C::M16) && size != 2) && !(C::BM > 128 && skv < (C::PV8 ? 2048 : C::QK8 ? 0 : 1152));
+                                : (C::QK8 && C::BM > 128 ? fills256 : !((C::BM > 128 || C::M16) && size != 2)) &&
+                                      !(C::BM > 128 && skv < (C::PV8 ? 2048 : C::QK8 ? 0 : 1152));
     if (C::KSPLIT ? (w.bm ? C::BM != w.bm : size != 0) : (w.bm ? C::BM != w.bm : !by_size)) return;
     if (w.bn && C::BN * C::SUB != w.bn) return;
     if (w.mfma && (C::M16 ? 16 : 32) != w.mfma) return;

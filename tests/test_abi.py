@@ -171,6 +171,11 @@ def test_predictable_latency_option_changes_the_choice_of_kernel_without_gpu():
     assert f.fmha_forward_kernel(f.CFK_FP16, 8, 32, 2048, 1216, 128) == "fmha_fwd_kernel16<128,64,8,2,0,0,0,0,1,0,1,0>"
     assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 8, 32, 2048, 1024, 128) == "fmha_fwd_kernel<128,64,4,2,1,1,0,0,1,0,0,0>"
     assert f.fmha_forward_kernel(f.CFK_FP8_E4M3, 8, 32, 2048, 2048, 128) == "fmha_fwd_kernel<128,64,8,2,1,1,0,0,2,0,0,0>"
+    # the compiler-scheduled 256-row builds for e4m3 Q and K (one 8-wave workgroup per CU) while their rounds of 256 items fill
+    hyb = lambda h: f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, h, 4096, 4096, 128, v_dtype=f.CFK_FP16).split(",")[2]
+    assert [hyb(h) for h in (8, 10, 16, 20, 24, 32, 36, 48)] == ["4", "8", "8", "4", "4", "8", "4", "8"]
+    e4 = lambda h: f.fmha_forward_kernel(f.CFK_FP8_E4M3, 1, h, 2048, 2048, 128).split(",")[2]
+    assert [e4(h) for h in (16, 20, 32, 40, 64, 72)] == ["4", "8", "8", "4", "8", "4"]
     # query lengths that leave the last 256-row tile partly filled: the 8-wave shape while at most a quarter of the rows idle
     assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 2016, 2048, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
     assert f.fmha_forward_kernel(f.CFK_FP16, 8, 16, 384, 2048, 128) == "fmha_fwd_kernel16p<128,64,8,2,0,0,0,0,2,0,1,1>"
